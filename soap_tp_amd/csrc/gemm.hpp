@@ -1,0 +1,391 @@
+// LDS-tiled MFMA GEMM for gfx950, column-major operands, fp32 (v_mfma_f32_32x32x2_f32) and
+// fp64 (v_mfma_f64_16x16x4_f64).  One kernel template serves every matrix product on the SOAP
+// path; what differs per call site is the epilogue functor, which receives each accumulator
+// element together with its global (m, n) coordinate:
+//   EpiStore     C = alpha*acc + beta*C                    (rotations, P*Q, block reflectors)
+//   EpiEmaLower  C = lerp(C, acc, w) on the lower triangle (Gram EMA, optional mirror)
+//   EpiAdam      Adam moment update + normalised update    (forward rotation, 2nd product)
+//   EpiPartial   raw partial sums for split-K              (tall-skinny products)
+//
+// Data layout.  op(A) is M x K, op(B) is K x N, both stored column-major with a leading
+// dimension; "trans" means the stored matrix is the transpose of the operand.  A K-slab of
+// each operand is staged in LDS as S[k][x] (x = m or n contiguous), so that the MFMA fragment
+// reads of a wavefront are 32 (16) consecutive words.  The MFMA "a" operand is fed from the
+// B tile and the "b" operand from the A tile: accumulator lanes then run along m, and every
+// epilogue load/store instruction touches 128 consecutive bytes of a column of C.
+#pragma once
+#include "common.hpp"
+
+namespace soapmi {
+
+template <typename T>
+struct GemmProblem {
+  const T* A;
+  const T* B;
+  int64_t lda, ldb;
+  int M, N, K;
+  int transA, transB;
+  int vecA, vecB;      // 16-byte global loads are legal for this operand
+  int tiles_m, tiles_n;
+  int num_tiles;
+  int lower;           // enumerate only tiles with tile_m >= tile_n (square tile grid)
+  int k_chunk;         // K extent handled by one blockIdx.y slice (multiple of BK)
+};
+
+// ---- epilogues ---------------------------------------------------------------------------
+template <typename T>
+struct EpiStore {
+  T* C;
+  int64_t ldc;
+  T alpha, beta;
+  __device__ __forceinline__ void operator()(int m, int n, T v, int) const {
+    T* p = C + m + (int64_t)n * ldc;
+    T r = alpha * v;
+    if (beta != T(0)) r += beta * (*p);
+    *p = r;
+  }
+};
+
+template <typename T>
+struct EpiPartial {
+  T* part;        // [splits][N][M] compact
+  int64_t ld;     // = M
+  int64_t slab;   // = M*N
+  __device__ __forceinline__ void operator()(int m, int n, T v, int z) const {
+    part[(int64_t)z * slab + m + (int64_t)n * ld] = v;
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ T lerp_like_torch(T start, T end, T weight) {
+  // Same two-branch form as torch.lerp (used by the reference: preconditioners.py:367,579).
+  return (weight < T(0.5)) ? start + weight * (end - start) : end - (end - start) * (T(1) - weight);
+}
+
+template <typename T>
+struct EpiEmaLower {
+  T* C;
+  int64_t ldc;
+  T weight;    // 1 - beta
+  int mirror;  // also write the transposed element so both triangles stay valid
+  __device__ __forceinline__ void operator()(int m, int n, T v, int) const {
+    if (m < n) return;
+    T* p = C + m + (int64_t)n * ldc;
+    T r = lerp_like_torch(*p, v, weight);
+    *p = r;
+    if (mirror && m != n) C[n + (int64_t)m * ldc] = r;
+  }
+};
+
+struct AdamScalars {
+  float beta1, beta2;
+  float one_minus_beta1, one_minus_beta2;
+  float bias_correction1;       // 1 - beta1^step
+  float sqrt_bias_correction2;  // sqrt(1 - beta2^step)
+  float eps;                    // already rescaled by the caller (soap.py:367)
+};
+
+__device__ __forceinline__ float adam_element(float g, float* mom, float* var, const AdamScalars& s) {
+  // Operation order follows optimizer.py:36-44.
+  float m = (*mom) * s.beta1 + g * s.one_minus_beta1;
+  float v = (*var) * s.beta2 + s.one_minus_beta2 * g * g;
+  *mom = m;
+  *var = v;
+  float denom = sqrtf(v) / s.sqrt_bias_correction2 + s.eps;
+  return (1.0f / denom) * m / s.bias_correction1;
+}
+
+struct EpiAdam {
+  float* mom;
+  float* var;
+  float* upd;
+  int64_t ldm, ldv, ldu;
+  AdamScalars s;
+  __device__ __forceinline__ void operator()(int m, int n, float g, int) const {
+    upd[m + (int64_t)n * ldu] = adam_element(g, mom + m + (int64_t)n * ldm, var + m + (int64_t)n * ldv, s);
+  }
+};
+
+// ---- kernel ------------------------------------------------------------------------------
+template <typename T, int BM_, int BN_, int BK_, int WM_, int WN_>
+struct GemmTile {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+  static constexpr int NT = 64 * WM * WN;
+  static constexpr int MI = Mfma<T>::MI, KI = Mfma<T>::KI;
+  static constexpr int TM = BM / WM / MI, TN = BN / WN / MI;
+  static constexpr int VW = Vec16<T>::W;
+  static constexpr int PAD = VW;  // keeps rows 16-byte aligned, skews banks for transposed stores
+  static constexpr int SA = BM + PAD, SB = BN + PAD;
+  static constexpr int NVA = BK * BM / VW / NT, NVB = BK * BN / VW / NT;
+  static_assert(BM % (WM * MI) == 0 && BN % (WN * MI) == 0, "wave tiling");
+  static_assert(BK % KI == 0 && BK % VW == 0, "k tiling");
+  static_assert((BK * BM / VW) % NT == 0 && (BK * BN / VW) % NT == 0, "loader tiling");
+};
+
+// Load one K-slab of an operand into registers.  X is the non-K extent (M for A, N for B).
+// xcontig: element (x, k) lives at base[x + k*ld]; otherwise at base[k + x*ld].
+template <typename T, int BX, int BK, int NT, int NV>
+__device__ __forceinline__ void load_slab(T (&reg)[NV][Vec16<T>::W], const T* __restrict__ base, int64_t ld,
+                                          int x0, int X, int k0, int kend, bool xcontig, bool vec, int tid) {
+  constexpr int VW = Vec16<T>::W;
+  using V = typename Vec16<T>::type;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    int v = tid + i * NT;
+    if (xcontig) {
+      int k = v / (BX / VW), xv = v % (BX / VW);
+      int gx = x0 + xv * VW, gk = k0 + k;
+      const T* p = base + gx + (int64_t)gk * ld;
+      if (vec) {
+        if (gx < X && gk < kend) {
+          V t = *reinterpret_cast<const V*>(p);
+          const T* tp = reinterpret_cast<const T*>(&t);
+#pragma unroll
+          for (int e = 0; e < VW; ++e) reg[i][e] = tp[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < VW; ++e) reg[i][e] = T(0);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VW; ++e) reg[i][e] = (gx + e < X && gk < kend) ? p[e] : T(0);
+      }
+    } else {
+      int x = v / (BK / VW), kv = v % (BK / VW);
+      int gx = x0 + x, gk = k0 + kv * VW;
+      const T* p = base + gk + (int64_t)gx * ld;
+      if (vec) {
+        if (gx < X && gk < kend) {
+          V t = *reinterpret_cast<const V*>(p);
+          const T* tp = reinterpret_cast<const T*>(&t);
+#pragma unroll
+          for (int e = 0; e < VW; ++e) reg[i][e] = tp[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < VW; ++e) reg[i][e] = T(0);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VW; ++e) reg[i][e] = (gx < X && gk + e < kend) ? p[e] : T(0);
+      }
+    }
+  }
+}
+
+template <typename T, int BX, int BK, int NT, int NV, int STRIDE>
+__device__ __forceinline__ void store_slab(T* __restrict__ S, const T (&reg)[NV][Vec16<T>::W], bool xcontig, int tid) {
+  constexpr int VW = Vec16<T>::W;
+  using V = typename Vec16<T>::type;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    int v = tid + i * NT;
+    if (xcontig) {
+      int k = v / (BX / VW), xv = v % (BX / VW);
+      V t;
+      T* tp = reinterpret_cast<T*>(&t);
+#pragma unroll
+      for (int e = 0; e < VW; ++e) tp[e] = reg[i][e];
+      *reinterpret_cast<V*>(S + k * STRIDE + xv * VW) = t;
+    } else {
+      int x = v / (BK / VW), kv = v % (BK / VW);
+#pragma unroll
+      for (int e = 0; e < VW; ++e) S[(kv * VW + e) * STRIDE + x] = reg[i][e];
+    }
+  }
+}
+
+template <typename T, class Cfg, class Epi>
+__global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi) {
+  using MF = Mfma<T>;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
+  constexpr int MI = Cfg::MI, KI = Cfg::KI, TM = Cfg::TM, TN = Cfg::TN;
+  constexpr int SA = Cfg::SA, SB = Cfg::SB, VW = Cfg::VW;
+
+  __shared__ __attribute__((aligned(16))) T As[2][BK * SA];
+  __shared__ __attribute__((aligned(16))) T Bs[2][BK * SB];
+
+  // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each XCD one
+  // contiguous range of tiles so that neighbouring tiles share its L2.
+  const int chunk = (p.num_tiles + 7) >> 3;
+  const int t = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+  if (t >= p.num_tiles) return;
+
+  int tm, tn;
+  if (p.lower) {
+    int bi = (int)((sqrtf(8.0f * (float)t + 1.0f) - 1.0f) * 0.5f);
+    while (bi * (bi + 1) / 2 > t) --bi;
+    while ((bi + 1) * (bi + 2) / 2 <= t) ++bi;
+    tm = bi;
+    tn = t - bi * (bi + 1) / 2;
+  } else {
+    const int per = 8 * p.tiles_n;
+    const int g = t / per, r = t - g * per;
+    const int rows = min(8, p.tiles_m - g * 8);
+    tm = g * 8 + r % rows;
+    tn = r / rows;
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int z = blockIdx.y;
+  const int kbeg = z * p.k_chunk;
+  const int kend = min(p.K, kbeg + p.k_chunk);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave % Cfg::WM) * (TM * MI);
+  const int wn0 = (wave / Cfg::WM) * (TN * MI);
+
+  typename MF::Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < MF::NACC; ++r) acc[i][j][r] = T(0);
+
+  T ra[Cfg::NVA][VW], rb[Cfg::NVB][VW];
+  const bool a_xc = !p.transA, b_xc = (p.transB != 0);
+  const int nk = (kend - kbeg + BK - 1) / BK;
+
+  if (nk > 0) {
+    load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, kbeg, kend, a_xc, p.vecA, tid);
+    load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, kbeg, kend, b_xc, p.vecB, tid);
+    store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[0], ra, a_xc, tid);
+    store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[0], rb, b_xc, tid);
+  }
+  __syncthreads();
+
+  const int krow = lane / MI, idx = lane % MI;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) {
+      const int k0 = kbeg + (kt + 1) * BK;
+      load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, k0, kend, a_xc, p.vecA, tid);
+      load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, k0, kend, b_xc, p.vecB, tid);
+    }
+    const T* as = As[buf];
+    const T* bs = Bs[buf];
+#pragma unroll
+    for (int kk = 0; kk < BK / KI; ++kk) {
+      T fm[TM], fn[TN];
+      const int kr = kk * KI + krow;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fm[i] = as[kr * SA + wm0 + i * MI + idx];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fn[j] = bs[kr * SB + wn0 + j * MI + idx];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(fn[j], fm[i], acc[i][j]);
+    }
+    if (kt + 1 < nk) {
+      store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[buf ^ 1], ra, a_xc, tid);
+      store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[buf ^ 1], rb, b_xc, tid);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm0 + i * MI + idx;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int r = 0; r < MF::NACC; ++r) {
+        const int n = n0 + wn0 + j * MI + MF::acc_row(r, lane);
+        if (m < p.M && n < p.N) epi(m, n, acc[i][j][r], z);
+      }
+    }
+  }
+}
+
+// Sum split-K partials and apply alpha/beta.
+template <typename T>
+__global__ void reduce_partials_kernel(const T* __restrict__ part, int splits, int64_t slab, int M, int N, T* C,
+                                       int64_t ldc, T alpha, T beta) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)M * N) return;
+  int m = (int)(i % M), n = (int)(i / M);
+  T s = T(0);
+  for (int z = 0; z < splits; ++z) s += part[(int64_t)z * slab + i];
+  T* p = C + m + (int64_t)n * ldc;
+  T r = alpha * s;
+  if (beta != T(0)) r += beta * (*p);
+  *p = r;
+}
+
+// ---- host side -----------------------------------------------------------------------------
+template <typename T>
+struct DefaultTile;
+template <>
+struct DefaultTile<float> {
+  using type = GemmTile<float, 128, 128, 16, 2, 2>;
+};
+template <>
+struct DefaultTile<double> {
+  using type = GemmTile<double, 128, 128, 8, 2, 2>;
+};
+
+template <typename T>
+static inline bool vec_ok(const T* p, int64_t ld, int contig_extent) {
+  constexpr int VW = Vec16<T>::W;
+  return (reinterpret_cast<uintptr_t>(p) % 16 == 0) && (ld % VW == 0) && (contig_extent % VW == 0);
+}
+
+template <typename T>
+static inline GemmProblem<T> make_problem(int transA, int transB, int M, int N, int K, const T* A, int64_t lda,
+                                          const T* B, int64_t ldb, bool lower) {
+  using Cfg = typename DefaultTile<T>::type;
+  GemmProblem<T> p;
+  p.A = A; p.B = B; p.lda = lda; p.ldb = ldb;
+  p.M = M; p.N = N; p.K = K;
+  p.transA = transA; p.transB = transB;
+  // contiguous extent: A not transposed -> m, transposed -> k ; B not transposed -> k, transposed -> n
+  p.vecA = vec_ok(A, lda, transA ? K : M);
+  p.vecB = vec_ok(B, ldb, transB ? N : K);
+  p.tiles_m = (int)ceil_div64(M, Cfg::BM);
+  p.tiles_n = (int)ceil_div64(N, Cfg::BN);
+  p.lower = lower ? 1 : 0;
+  p.num_tiles = lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
+  p.k_chunk = (int)(ceil_div64(K > 0 ? K : 1, Cfg::BK) * Cfg::BK);
+  return p;
+}
+
+template <typename T, class Epi>
+static inline int launch_gemm(hipStream_t stream, const GemmProblem<T>& p, const Epi& epi, int k_splits = 1) {
+  using Cfg = typename DefaultTile<T>::type;
+  if (p.M <= 0 || p.N <= 0) return kOk;
+  const int chunk = (p.num_tiles + 7) / 8;
+  dim3 grid(8 * chunk, k_splits, 1);
+  hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi>), grid, dim3(Cfg::NT), 0, stream, p, epi);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
+// C = alpha*op(A)*op(B) + beta*C.  If `partials` is non-null and k_splits > 1 the K range is
+// cut into k_splits slices whose partial products are summed by a second kernel (fixed
+// order, so the result does not depend on scheduling).
+template <typename T>
+static inline int gemm(hipStream_t stream, int transA, int transB, int M, int N, int K, T alpha, const T* A,
+                       int64_t lda, const T* B, int64_t ldb, T beta, T* C, int64_t ldc, int k_splits = 1,
+                       T* partials = nullptr) {
+  using Cfg = typename DefaultTile<T>::type;
+  if (M <= 0 || N <= 0) return kOk;
+  GemmProblem<T> p = make_problem<T>(transA, transB, M, N, K, A, lda, B, ldb, false);
+  if (k_splits > 1 && partials != nullptr && K > Cfg::BK) {
+    int64_t slabs = ceil_div64(K, Cfg::BK);
+    p.k_chunk = (int)(ceil_div64(slabs, k_splits) * Cfg::BK);
+    int splits = (int)ceil_div64(K, p.k_chunk);
+    EpiPartial<T> ep{partials, (int64_t)M, (int64_t)M * N};
+    int rc = launch_gemm<T>(stream, p, ep, splits);
+    if (rc) return rc;
+    int64_t total = (int64_t)M * N;
+    hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3((unsigned)ceil_div64(total, 256)), dim3(256), 0, stream,
+                       partials, splits, (int64_t)M * N, M, N, C, ldc, alpha, beta);
+    SOAPMI_LAUNCH_CHECK();
+    return kOk;
+  }
+  EpiStore<T> ep{C, ldc, alpha, beta};
+  return launch_gemm<T>(stream, p, ep, 1);
+}
+
+}  // namespace soapmi
