@@ -106,6 +106,90 @@ int soapmi_row_major_to_col_major_f32(const float* in, int64_t ldi, float* out, 
 int soapmi_col_major_to_row_major_f32(const float* in, int64_t ldi, float* out, int64_t ldo, int64_t rows,
                                       int64_t cols, void* stream);
 
+/* ---- basis refresh ------------------------------------------------------------------------ */
+
+/* work <- A Q for the symmetric n x n matrix A (both triangles must be valid).  Replaces
+ * slate_symmetric_multiply_float (src/soap_tp/csrc/slate_bindings.cpp:55-123), which on GPU
+ * builds is a plain product with the full matrix (:113-116). */
+int soapmi_symm_f32(const float* a, const float* q, float* work, int64_t n, int64_t lda, int64_t ldq, int64_t ldw,
+                    void* stream);
+
+/* estimates[j] = sum_i q[i, j] * work[i, j]: diag(Q^T P Q) once work = P Q
+ * (src/soap_tp/ops/factorizations.py:255-257).  Fixed-order reduction. */
+int soapmi_column_dots_f32(const float* q, int64_t ldq, const float* work, int64_t ldw, int64_t rows, int64_t cols,
+                           float* estimates, void* stream);
+
+/* order <- argsort(keys, descending) as int64 (factorizations.py:271).  Ties are broken by the
+ * smaller index, NaNs sort last.  Workspace is only used above 16384 keys. */
+int soapmi_argsort_desc_f32(const float* keys, int64_t n, int64_t* order, void* workspace, size_t workspace_bytes,
+                            void* stream);
+size_t soapmi_argsort_workspace_bytes(int64_t n);
+
+/* out[i, j] = in[row_order[i], col_order[j]]; a NULL order is the identity; out must not overlap in. */
+int soapmi_gather_f32(const float* in, int64_t ldi, float* out, int64_t ldo, int64_t rows, int64_t cols,
+                      const int64_t* row_order, const int64_t* col_order, void* stream);
+
+/* In-place matrix <- matrix[row_order][:, col_order]; replaces permute_2d_block_cyclic_
+ * (src/soap_tp/ops/optimizer.py:395-567).  Workspace: rows*cols floats. */
+int soapmi_permute_f32(float* matrix, int64_t ld, int64_t rows, int64_t cols, const int64_t* row_order,
+                       const int64_t* col_order, void* workspace, size_t workspace_bytes, void* stream);
+size_t soapmi_permute_workspace_bytes(int64_t rows, int64_t cols);
+
+/* Returns 1 if order[0..n) is a permutation of range(n), 0 if not, <0 on error
+ * (optimizer.py:47-61).  Synchronises the stream.  Workspace: (n + 1) ints. */
+int soapmi_is_permutation(const int64_t* order, int64_t n, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Householder QR of the n x n `matrix` (destroyed), explicit orthogonal factor into `q`.
+ * Replaces slate_qr_float (src/soap_tp/csrc/slate_bindings.cpp:125-189: geqrf, set Q = I,
+ * unmqr); same LAPACK sign convention (diagonal of R opposite in sign to the pivot). */
+int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t ldq, void* workspace,
+                  size_t workspace_bytes, void* stream);
+size_t soapmi_qr_workspace_bytes(int64_t n);
+
+/* One power iteration and QR for one basis (power_iteration_qr_2d_block_cyclic_,
+ * src/soap_tp/ops/factorizations.py:323-360): work = P Q, estimates = column dots,
+ * order = argsort(descending), work = work[:, order], Q = qr(work).Q.
+ * symmetrize != 0 first copies P's lower triangle onto its upper one (for P maintained by
+ * soapmi_gram_ema_f32 with mirror == 0).  `estimates` may be NULL. */
+int soapmi_power_iteration_qr_f32(float* p, float* q, float* work, int64_t n, int64_t ldp, int64_t ldq,
+                                  int64_t ldw, int symmetrize, int64_t* order, float* estimates, void* workspace,
+                                  size_t workspace_bytes, void* stream);
+size_t soapmi_power_iteration_qr_workspace_bytes(int64_t n);
+
+/* refresh_bases_and_transport_optimizer_state_ (src/soap_tp/ops/factorizations.py:550-614):
+ * momentum to parameter space with the old bases, power iteration + QR on both sides, variance
+ * <- variance[left_order][:, right_order], momentum into the new bases. */
+int soapmi_refresh_f32(float* momentum, int64_t ldm, float* variance, int64_t ldv, float* left_preconditioner,
+                       int64_t ldl, float* right_preconditioner, int64_t ldr, float* q_left, int64_t ldql,
+                       float* q_right, int64_t ldqr, float* left_work, int64_t ldlw, float* right_work,
+                       int64_t ldrw, int64_t rows, int64_t cols, int symmetrize, int64_t* left_order,
+                       int64_t* right_order, void* workspace, size_t workspace_bytes, void* stream);
+size_t soapmi_refresh_workspace_bytes(int64_t rows, int64_t cols);
+
+/* ---- symmetric eigensolver (basis initialisation) ------------------------------------------ */
+
+/* All eigenpairs of the symmetric n x n matrix `a` (lower triangle referenced, contents
+ * destroyed): eigenvalues ascending into `eigenvalues`, eigenvectors into the columns of `q`.
+ * Replaces elpa_eigenvectors_2d_block_cyclic_double / initialize_basis_2d_block_cyclic_ of the
+ * ELPA module (src/soap_tp/csrc/elpa_bindings.cpp:61-196, alias :234-235; one-stage solver, nev = n,
+ * ascending, input destroyed) on a 1x1 grid, where local_rows == lda == n.  Householder
+ * tridiagonalisation, divide and conquer, back-transformation; no host synchronisation. */
+int soapmi_eigh_f64(double* a, double* eigenvalues, double* q, int64_t n, int64_t lda, int64_t ldq,
+                    void* workspace, size_t workspace_bytes, void* stream);
+int soapmi_eigh_f32(float* a, float* eigenvalues, float* q, int64_t n, int64_t lda, int64_t ldq, void* workspace,
+                    size_t workspace_bytes, void* stream);
+size_t soapmi_eigh_workspace_bytes(int64_t n, int element_bytes);
+
+/* Descending eigenbasis of the preconditioner P into Q, eigenvalues (descending, float) into
+ * `eigenvalues`: initialize_basis_2d_block_cyclic_ (src/soap_tp/ops/factorizations.py:363-547) on a
+ * 1x1 grid.  implementation 0 ("elpa", :472-547): work <- -P, float64 copies, ascending solve of
+ * -P, Q = float(Q64), eigenvalues = -lambda.  implementation 1 ("eigh", :421-470): float32 solve
+ * of P + 1e-30 I, columns and eigenvalues flipped.  Only the lower triangle of P is read. */
+int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* eigenvalues, int64_t n, int64_t ldp,
+                                int64_t ldq, int64_t ldw, int implementation, void* workspace,
+                                size_t workspace_bytes, void* stream);
+size_t soapmi_initialize_basis_workspace_bytes(int64_t n, int implementation);
+
 #ifdef __cplusplus
 }
 #endif

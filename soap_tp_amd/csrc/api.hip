@@ -5,8 +5,11 @@
 
 #include "../../include/soap_mi355.h"
 #include "common.hpp"
+#include "eigh.hpp"
 #include "elementwise.hpp"
 #include "gemm.hpp"
+#include "qr.hpp"
+#include "refresh.hpp"
 
 namespace soapmi {
 
@@ -82,6 +85,27 @@ static int check_adam_args(int64_t step, double beta1, double beta2, double eps)
 }  // namespace soapmi
 
 using namespace soapmi;
+
+static int resolve_workspace_fwd(void* user, size_t user_bytes, size_t need, void** out) {
+  return resolve_workspace(user, user_bytes, need, out);
+}
+
+template <typename T>
+static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_t ldq, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  SOAPMI_REQUIRE(a && eigenvalues && q, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(n > 0, "matrix dimensions and block size must be positive");
+  SOAPMI_REQUIRE(lda >= n && ldq >= n, "leading dimensions are too small");
+  SOAPMI_REQUIRE(n <= 32768, "matrix size %lld exceeds the supported maximum 32768", (long long)n);
+  const size_t need = eigh_workspace_bytes<T>(n);
+  void* ws = nullptr;
+  int rc = resolve_workspace_fwd(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  Workspace w(ws, need);
+  EighWorkspace<T> ews;
+  eigh_workspace_layout<T>(w, n, &ews);
+  return eigh_ascending<T>((hipStream_t)stream, a, lda, eigenvalues, q, ldq, (int)n, ews);
+}
 
 extern "C" {
 
@@ -258,6 +282,328 @@ int soapmi_col_major_to_row_major_f32(const float* in, int64_t ldi, float* out, 
   SOAPMI_REQUIRE(ldi >= rows && ldo >= cols, "leading dimensions are too small");
   hipLaunchKernelGGL((transpose_kernel<float>), dim3((unsigned)ceil_div64(rows, 64), (unsigned)ceil_div64(cols, 64)),
                      dim3(256), 0, (hipStream_t)stream, in, ldi, out, ldo, (int)rows, (int)cols);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
+
+// ---- basis refresh ---------------------------------------------------------------------------
+
+int soapmi_symm_f32(const float* a, const float* q, float* work, int64_t n, int64_t lda, int64_t ldq, int64_t ldw,
+                    void* stream) {
+  SOAPMI_REQUIRE(a && q && work, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(n > 0 && lda >= n && ldq >= n && ldw >= n, "matrix size and leading dimensions must be positive");
+  return gemm<float>((hipStream_t)stream, 0, 0, (int)n, (int)n, (int)n, 1.0f, a, lda, q, ldq, 0.0f, work, ldw);
+}
+
+int soapmi_column_dots_f32(const float* q, int64_t ldq, const float* work, int64_t ldw, int64_t rows, int64_t cols,
+                           float* estimates, void* stream) {
+  SOAPMI_REQUIRE(rows >= 0 && cols >= 0, "matrix dimensions must be non-negative");
+  if (cols == 0) return kOk;
+  SOAPMI_REQUIRE(q && work && estimates, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(ldq >= rows && ldw >= rows, "leading dimensions are too small");
+  hipLaunchKernelGGL((coldot_kernel<float>), dim3((unsigned)cols), dim3(256), 0, (hipStream_t)stream, q, ldq, work, ldw,
+                     (int)rows, estimates);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
+static int next_pow2(int64_t n) {
+  int p = 1;
+  while (p < n) p <<= 1;
+  return p;
+}
+constexpr int kArgsortLdsMax = 16384;
+
+size_t soapmi_argsort_workspace_bytes(int64_t n) {
+  const int np2 = next_pow2(n);
+  WorkspaceSizer w;
+  if (np2 > kArgsortLdsMax) {
+    w.take<float>((size_t)np2);
+    w.take<int>((size_t)np2);
+  }
+  return w.total();
+}
+
+int soapmi_argsort_desc_f32(const float* keys, int64_t n, int64_t* order, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+  SOAPMI_REQUIRE(n >= 0 && n < (1 << 30), "key count out of range");
+  if (n == 0) return kOk;
+  SOAPMI_REQUIRE(keys && order, "buffer addresses must be nonzero");
+  hipStream_t s = (hipStream_t)stream;
+  const int np2 = next_pow2(n);
+  if (np2 <= kArgsortLdsMax) {
+    const size_t lds = (size_t)np2 * (sizeof(float) + sizeof(int));
+    static bool attribute_set = false;
+    if (!attribute_set) {
+      SOAPMI_HIP(hipFuncSetAttribute((const void*)argsort_desc_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     kArgsortLdsMax * 8));
+      attribute_set = true;
+    }
+    const int threads = np2 >= 2048 ? 1024 : (np2 >= 128 ? np2 / 2 : 64);
+    hipLaunchKernelGGL(argsort_desc_lds_kernel, dim3(1), dim3(threads), lds, s, keys, (int)n, np2, order);
+    SOAPMI_LAUNCH_CHECK();
+    return kOk;
+  }
+  const size_t need = soapmi_argsort_workspace_bytes(n);
+  void* ws = nullptr;
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  Workspace w(ws, need);
+  float* v = w.take<float>((size_t)np2);
+  int* id = w.take<int>((size_t)np2);
+  const unsigned blocks = (unsigned)ceil_div64(np2, 256);
+  hipLaunchKernelGGL(argsort_init_kernel, dim3(blocks), dim3(256), 0, s, keys, (int)n, np2, v, id);
+  for (int k = 2; k <= np2; k <<= 1)
+    for (int j = k >> 1; j > 0; j >>= 1)
+      hipLaunchKernelGGL(argsort_stage_kernel, dim3(blocks), dim3(256), 0, s, v, id, np2, k, j);
+  hipLaunchKernelGGL(argsort_finish_kernel, dim3((unsigned)ceil_div64(n, 256)), dim3(256), 0, s, id, (int)n, order);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
+static inline dim3 grid_rows_cols(int64_t rows, int64_t cols) {
+  return dim3((unsigned)ceil_div64(rows, 256), (unsigned)(cols < 8192 ? (cols > 0 ? cols : 1) : 8192));
+}
+
+int soapmi_gather_f32(const float* in, int64_t ldi, float* out, int64_t ldo, int64_t rows, int64_t cols,
+                      const int64_t* row_order, const int64_t* col_order, void* stream) {
+  SOAPMI_REQUIRE(rows >= 0 && cols >= 0, "matrix dimensions must be non-negative");
+  if (rows == 0 || cols == 0) return kOk;
+  SOAPMI_REQUIRE(in && out && in != out, "buffers must be nonzero and distinct");
+  SOAPMI_REQUIRE(ldi >= rows && ldo >= rows, "leading dimensions are too small");
+  hipLaunchKernelGGL((gather2d_kernel<float>), grid_rows_cols(rows, cols), dim3(256), 0, (hipStream_t)stream, in, ldi,
+                     out, ldo, (int)rows, (int)cols, row_order, col_order);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
+size_t soapmi_permute_workspace_bytes(int64_t rows, int64_t cols) {
+  WorkspaceSizer w;
+  w.take<float>((size_t)rows * cols);
+  return w.total();
+}
+
+static int permute_with(hipStream_t s, float* matrix, int64_t ld, int64_t rows, int64_t cols,
+                        const int64_t* row_order, const int64_t* col_order, float* tmp) {
+  hipLaunchKernelGGL((gather2d_kernel<float>), grid_rows_cols(rows, cols), dim3(256), 0, s, matrix, ld, tmp, rows,
+                     (int)rows, (int)cols, row_order, col_order);
+  hipLaunchKernelGGL((copy2d_kernel<float>), grid_rows_cols(rows, cols), dim3(256), 0, s, tmp, rows, matrix, ld,
+                     (int)rows, (int)cols);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
+int soapmi_permute_f32(float* matrix, int64_t ld, int64_t rows, int64_t cols, const int64_t* row_order,
+                       const int64_t* col_order, void* workspace, size_t workspace_bytes, void* stream) {
+  SOAPMI_REQUIRE(rows >= 0 && cols >= 0, "matrix dimensions must be non-negative");
+  if (rows == 0 || cols == 0) return kOk;
+  SOAPMI_REQUIRE(matrix, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(ld >= rows, "leading dimension is too small");
+  const size_t need = soapmi_permute_workspace_bytes(rows, cols);
+  void* ws = nullptr;
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  Workspace w(ws, need);
+  float* tmp = w.take<float>((size_t)rows * cols);
+  return permute_with((hipStream_t)stream, matrix, ld, rows, cols, row_order, col_order, tmp);
+}
+
+int soapmi_is_permutation(const int64_t* order, int64_t n, void* workspace, size_t workspace_bytes, void* stream) {
+  SOAPMI_REQUIRE(n >= 0 && n < (1ll << 31), "size out of range");
+  if (n == 0) return 1;
+  SOAPMI_REQUIRE(order, "buffer addresses must be nonzero");
+  const size_t need = (size_t)(n + 1) * sizeof(int) + 512;
+  void* ws = nullptr;
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  int* seen = static_cast<int*>(ws);
+  int* flag = seen + n;
+  SOAPMI_HIP(hipMemsetAsync(seen, 0, (size_t)(n + 1) * sizeof(int), s));
+  hipLaunchKernelGGL(check_permutation_kernel, dim3((unsigned)ceil_div64(n, 256)), dim3(256), 0, s, order, (int)n, seen,
+                     flag);
+  SOAPMI_LAUNCH_CHECK();
+  int host_flag = 0;
+  SOAPMI_HIP(hipMemcpyAsync(&host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, s));
+  SOAPMI_HIP(hipStreamSynchronize(s));
+  return host_flag ? 0 : 1;
+}
+
+size_t soapmi_qr_workspace_bytes(int64_t n) { return qr_workspace_bytes<float>(n); }
+
+int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t ldq, void* workspace,
+                  size_t workspace_bytes, void* stream) {
+  SOAPMI_REQUIRE(matrix && q, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(n > 0 && ldmatrix > 0 && ldq > 0, "matrix size and leading dimensions must be positive");
+  SOAPMI_REQUIRE(ldmatrix >= n && ldq >= n, "leading dimensions are too small");
+  SOAPMI_REQUIRE(matrix != q, "matrix and q must not overlap");
+  const size_t need = soapmi_qr_workspace_bytes(n);
+  void* ws = nullptr;
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  Workspace w(ws, need);
+  QrWorkspace<float> qws;
+  qr_workspace_layout<float>(w, n, &qws);
+  return qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws);
+}
+
+size_t soapmi_power_iteration_qr_workspace_bytes(int64_t n) {
+  WorkspaceSizer w;
+  w.take<float>((size_t)n * n);  // gather target
+  w.take<float>((size_t)n);      // estimates
+  w.take<char>(soapmi_argsort_workspace_bytes(n));
+  w.take<char>(soapmi_qr_workspace_bytes(n));
+  return w.total();
+}
+
+int soapmi_power_iteration_qr_f32(float* p, float* q, float* work, int64_t n, int64_t ldp, int64_t ldq,
+                                  int64_t ldw, int symmetrize, int64_t* order, float* estimates, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  SOAPMI_REQUIRE(p && q && work && order, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(n > 0 && ldp >= n && ldq >= n && ldw >= n, "matrix size and leading dimensions must be positive");
+  SOAPMI_REQUIRE(p != q && p != work && q != work, "preconditioner, Q, and work must not overlap.");
+  const size_t need = soapmi_power_iteration_qr_workspace_bytes(n);
+  void* ws = nullptr;
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  Workspace w(ws, need);
+  float* tmp = w.take<float>((size_t)n * n);
+  float* est = w.take<float>((size_t)n);
+  const size_t sort_bytes = soapmi_argsort_workspace_bytes(n);
+  char* sort_ws = w.take<char>(sort_bytes);
+  const size_t qr_bytes = soapmi_qr_workspace_bytes(n);
+  char* qr_ws = w.take<char>(qr_bytes);
+  hipStream_t s = (hipStream_t)stream;
+  if (symmetrize) {
+    rc = soapmi_symmetrize_lower_f32(p, n, ldp, stream);
+    if (rc) return rc;
+  }
+  rc = soapmi_symm_f32(p, q, work, n, ldp, ldq, ldw, stream);
+  if (rc) return rc;
+  rc = soapmi_column_dots_f32(q, ldq, work, ldw, n, n, est, stream);
+  if (rc) return rc;
+  if (estimates) SOAPMI_HIP(hipMemcpyAsync(estimates, est, (size_t)n * sizeof(float), hipMemcpyDeviceToDevice, s));
+  rc = soapmi_argsort_desc_f32(est, n, order, sort_ws, sort_bytes, stream);
+  if (rc) return rc;
+  rc = permute_with(s, work, ldw, n, n, nullptr, order, tmp);
+  if (rc) return rc;
+  return soapmi_qr_f32(work, q, n, ldw, ldq, qr_ws, qr_bytes, stream);
+}
+
+size_t soapmi_refresh_workspace_bytes(int64_t rows, int64_t cols) {
+  size_t a = soapmi_rotate_workspace_bytes(rows, cols);
+  size_t b = soapmi_power_iteration_qr_workspace_bytes(rows);
+  size_t c = soapmi_power_iteration_qr_workspace_bytes(cols);
+  size_t d = soapmi_permute_workspace_bytes(rows, cols);
+  size_t m = a > b ? a : b;
+  m = m > c ? m : c;
+  return m > d ? m : d;
+}
+
+int soapmi_refresh_f32(float* momentum, int64_t ldm, float* variance, int64_t ldv, float* left_preconditioner,
+                       int64_t ldl, float* right_preconditioner, int64_t ldr, float* q_left, int64_t ldql,
+                       float* q_right, int64_t ldqr, float* left_work, int64_t ldlw, float* right_work,
+                       int64_t ldrw, int64_t rows, int64_t cols, int symmetrize, int64_t* left_order,
+                       int64_t* right_order, void* workspace, size_t workspace_bytes, void* stream) {
+  SOAPMI_REQUIRE(momentum && variance && left_order && right_order, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(rows > 0 && cols > 0, "matrix dimensions must be positive");
+  const size_t need = soapmi_refresh_workspace_bytes(rows, cols);
+  void* ws = nullptr;
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  rc = soapmi_rotate_f32(q_left, momentum, q_right, rows, cols, ldql, ldm, ldqr, 0, ws, need, stream);
+  if (rc) return rc;
+  rc = soapmi_power_iteration_qr_f32(left_preconditioner, q_left, left_work, rows, ldl, ldql, ldlw, symmetrize,
+                                     left_order, nullptr, ws, need, stream);
+  if (rc) return rc;
+  rc = soapmi_power_iteration_qr_f32(right_preconditioner, q_right, right_work, cols, ldr, ldqr, ldrw, symmetrize,
+                                     right_order, nullptr, ws, need, stream);
+  if (rc) return rc;
+  rc = soapmi_permute_f32(variance, ldv, rows, cols, left_order, right_order, ws, need, stream);
+  if (rc) return rc;
+  return soapmi_rotate_f32(q_left, momentum, q_right, rows, cols, ldql, ldm, ldqr, 1, ws, need, stream);
+}
+
+
+// ---- eigensolver ------------------------------------------------------------------------------
+
+size_t soapmi_eigh_workspace_bytes(int64_t n, int element_bytes) {
+  return element_bytes == 8 ? eigh_workspace_bytes<double>(n) : eigh_workspace_bytes<float>(n);
+}
+
+int soapmi_eigh_f64(double* a, double* eigenvalues, double* q, int64_t n, int64_t lda, int64_t ldq,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+  return eigh_entry<double>(a, eigenvalues, q, n, lda, ldq, workspace, workspace_bytes, stream);
+}
+
+int soapmi_eigh_f32(float* a, float* eigenvalues, float* q, int64_t n, int64_t lda, int64_t ldq, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  return eigh_entry<float>(a, eigenvalues, q, n, lda, ldq, workspace, workspace_bytes, stream);
+}
+
+size_t soapmi_initialize_basis_workspace_bytes(int64_t n, int implementation) {
+  WorkspaceSizer w;
+  if (implementation == 0) {
+    w.take<double>((size_t)n * n);
+    w.take<double>((size_t)n * n);
+    w.take<double>((size_t)n);
+    w.take<char>(eigh_workspace_bytes<double>(n));
+  } else {
+    w.take<float>((size_t)n * n);
+    w.take<float>((size_t)n * n);
+    w.take<float>((size_t)n);
+    w.take<char>(eigh_workspace_bytes<float>(n));
+  }
+  return w.total();
+}
+
+int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* eigenvalues, int64_t n, int64_t ldp,
+                                int64_t ldq, int64_t ldw, int implementation, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  SOAPMI_REQUIRE(implementation == 0 || implementation == 1, "implementation must be 0 (elpa) or 1 (eigh), got %d.",
+                 implementation);
+  SOAPMI_REQUIRE(p && q && work && eigenvalues, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(n > 0, "matrix dimensions and block size must be positive");
+  SOAPMI_REQUIRE(ldp >= n && ldq >= n && ldw >= n, "leading dimensions are too small");
+  SOAPMI_REQUIRE(p != q && p != work && q != work, "preconditioner, Q, and work must not overlap.");
+  const size_t need = soapmi_initialize_basis_workspace_bytes(n, implementation);
+  void* ws = nullptr;
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  Workspace w(ws, need);
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)ceil_div64(n, 256), (unsigned)(n < 4096 ? n : 4096));
+  const unsigned vblocks = (unsigned)ceil_div64(n, 256);
+  if (implementation == 0) {
+    double* a64 = w.take<double>((size_t)n * n);
+    double* z64 = w.take<double>((size_t)n * n);
+    double* w64 = w.take<double>((size_t)n);
+    const size_t eb = eigh_workspace_bytes<double>(n);
+    char* ebuf = w.take<char>(eb);
+    // work <- -P (both triangles), then its float64 copy, as factorizations.py:500-507 stages them
+    hipLaunchKernelGGL((sym_convert_kernel<float, float>), grid, dim3(256), 0, s, p, ldp, work, ldw, (int)n, -1.0f, 0.0f);
+    hipLaunchKernelGGL((sym_convert_kernel<float, double>), grid, dim3(256), 0, s, p, ldp, a64, n, (int)n, -1.0, 0.0);
+    SOAPMI_LAUNCH_CHECK();
+    rc = soapmi_eigh_f64(a64, w64, z64, n, n, n, ebuf, eb, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL((convert_columns_kernel<double, float>), grid, dim3(256), 0, s, z64, n, q, ldq, (int)n, 0);
+    hipLaunchKernelGGL((convert_vector_kernel<double, float>), dim3(vblocks), dim3(256), 0, s, w64, eigenvalues, (int)n,
+                       -1.0f, 0);
+  } else {
+    float* a32 = w.take<float>((size_t)n * n);
+    float* z32 = w.take<float>((size_t)n * n);
+    float* w32 = w.take<float>((size_t)n);
+    const size_t eb = eigh_workspace_bytes<float>(n);
+    char* ebuf = w.take<char>(eb);
+    hipLaunchKernelGGL((sym_convert_kernel<float, float>), grid, dim3(256), 0, s, p, ldp, a32, n, (int)n, 1.0f, 1e-30f);
+    SOAPMI_LAUNCH_CHECK();
+    rc = soapmi_eigh_f32(a32, w32, z32, n, n, n, ebuf, eb, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL((convert_columns_kernel<float, float>), grid, dim3(256), 0, s, z32, n, q, ldq, (int)n, 1);
+    hipLaunchKernelGGL((convert_vector_kernel<float, float>), dim3(vblocks), dim3(256), 0, s, w32, eigenvalues, (int)n,
+                       1.0f, 1);
+  }
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }

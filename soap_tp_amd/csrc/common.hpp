@@ -68,7 +68,10 @@ struct Workspace {
 struct WorkspaceSizer {
   size_t used = 0;
   template <typename T>
-  void take(size_t count) { used = align_up(used, 256) + count * sizeof(T); }
+  T* take(size_t count) {
+    used = align_up(used, 256) + count * sizeof(T);
+    return nullptr;
+  }
   size_t total() const { return align_up(used, 256) + 256; }
 };
 

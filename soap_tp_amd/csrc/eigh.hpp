@@ -1,0 +1,117 @@
+// Dense symmetric eigensolver: tridiagonalise (sytrd.hpp), divide and conquer on the tridiagonal
+// matrix (stedc.hpp), back-transform the eigenvectors with the stored reflectors (compact-WY
+// blocks on the MFMA GEMM).  Same three stages as the one-stage ELPA solver the reference calls
+// (src/soap_tp/csrc/elpa_bindings.cpp:149,165); eigenvalues come back ascending.
+#pragma once
+#include "common.hpp"
+#include "elementwise.hpp"
+#include "gemm.hpp"
+#include "qr.hpp"
+#include "stedc.hpp"
+#include "sytrd.hpp"
+
+namespace soapmi {
+
+template <typename T>
+struct EighWorkspace {
+  T* d;
+  T* e;
+  T* tau;
+  TrdWorkspace<T> trd;
+  DcWorkspace<T> dc;
+  QrWorkspace<T> br;  // block-reflector scratch for the back-transformation
+};
+
+template <typename T, class WS>
+static inline void eigh_workspace_layout(WS& ws, int64_t n, EighWorkspace<T>* out) {
+  EighWorkspace<T> w;
+  w.d = ws.template take<T>(n);
+  w.e = ws.template take<T>(n);
+  w.tau = ws.template take<T>(n);
+  trd_workspace_layout<T>(ws, n, out ? &w.trd : nullptr);
+  dc_workspace_layout<T>(ws, n, out ? &w.dc : nullptr);
+  qr_workspace_layout<T>(ws, n, out ? &w.br : nullptr);
+  if (out) *out = w;
+}
+
+template <typename T>
+static inline size_t eigh_workspace_bytes(int64_t n) {
+  WorkspaceSizer sizer;
+  eigh_workspace_layout<T>(sizer, n, nullptr);
+  return sizer.total();
+}
+
+// A (n x n, lower triangle referenced, destroyed) = Z diag(w) Z^T, w ascending.
+template <typename T>
+static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, int64_t ldz, int n,
+                                 const EighWorkspace<T>& ws) {
+  if (n <= 0) return kOk;
+  {
+    const unsigned nb = (unsigned)ceil_div64(n, 64);
+    hipLaunchKernelGGL((symmetrize_lower_kernel<T>), dim3(nb, nb), dim3(256), 0, s, A, lda, n);
+    SOAPMI_LAUNCH_CHECK();
+  }
+  int rc = sytrd_lower<T>(s, A, lda, n, ws.d, ws.e, ws.tau, ws.trd);
+  if (rc) return rc;
+  rc = stedc<T>(s, n, ws.d, ws.e, w, Z, ldz, ws.dc);
+  if (rc) return rc;
+  // Z <- H_0 H_1 ... H_{n-2} Z, block reflectors applied last panel first.
+  const int nref = n - 1;  // reflector j lives in column j, rows j+1..n-1
+  if (nref <= 0) return kOk;
+  constexpr int NB = kQrNb;
+  const int panels = (int)ceil_div64(nref, NB);
+  const int64_t ldv = n;
+  for (int pi = panels - 1; pi >= 0; --pi) {
+    const int p = pi * NB, pe = std::min(nref, p + NB), nbw = pe - p;
+    const int rows = n - p - 1;
+    hipLaunchKernelGGL((extract_v_kernel<T>), dim3((unsigned)ceil_div64(rows, 256)), dim3(256), 0, s, A, lda, rows, p + 1,
+                       p, nbw, ws.br.vc, ldv);
+    SOAPMI_LAUNCH_CHECK();
+    const int splits = rows >= 2048 ? kQrSplits : 1;
+    rc = gemm<T, typename SkinnyTile<T>::type>(s, 1, 0, nbw, nbw, rows, T(1), ws.br.vc, ldv, ws.br.vc, ldv, T(0),
+                                               ws.br.gram, NB, splits, ws.br.splitk);
+    if (rc) return rc;
+    hipLaunchKernelGGL((larft_kernel<T>), dim3(1), dim3(64), 0, s, ws.br.gram, NB, ws.tau + p, nbw, ws.br.t_all, NB);
+    SOAPMI_LAUNCH_CHECK();
+    rc = apply_block_reflector<T>(s, ws.br, ws.br.t_all, false, rows, nbw, n, ldv, Z + (p + 1), ldz);
+    if (rc) return rc;
+  }
+  return kOk;
+}
+
+// out[i, j] = scale * (T_out) in[max(i,j), min(i,j)] (+ shift on the diagonal): builds the full
+// symmetric solver input from the lower triangle of P, converting precision on the way.
+template <typename Tin, typename Tout>
+__global__ void sym_convert_kernel(const Tin* __restrict__ in, int64_t ldi, Tout* __restrict__ out, int64_t ldo, int n,
+                                   Tout scale, Tout diag_shift) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  for (int j = blockIdx.y; j < n; j += gridDim.y) {
+    const int r = i > j ? i : j, c = i > j ? j : i;
+    Tout v = scale * (Tout)in[r + (int64_t)c * ldi];
+    if (i == j) v += diag_shift;
+    out[i + (int64_t)j * ldo] = v;
+  }
+}
+
+// out[i, j] = (Tout) in[i, reverse ? n-1-j : j]
+template <typename Tin, typename Tout>
+__global__ void convert_columns_kernel(const Tin* __restrict__ in, int64_t ldi, Tout* __restrict__ out, int64_t ldo,
+                                       int n, int reverse) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  for (int j = blockIdx.y; j < n; j += gridDim.y) {
+    const int sj = reverse ? n - 1 - j : j;
+    out[i + (int64_t)j * ldo] = (Tout)in[i + (int64_t)sj * ldi];
+  }
+}
+
+template <typename Tin, typename Tout>
+__global__ void convert_vector_kernel(const Tin* __restrict__ in, Tout* __restrict__ out, int n, Tout scale,
+                                      int reverse) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  out[i] = scale * (Tout)in[reverse ? n - 1 - i : i];
+}
+
+}  // namespace soapmi

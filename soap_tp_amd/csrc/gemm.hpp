@@ -195,7 +195,7 @@ __device__ __forceinline__ void store_slab(T* __restrict__ S, const T (&reg)[NV]
 }
 
 template <typename T, class Cfg, class Epi>
-__global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi) {
+__device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Epi& epi, const int wg, const int z) {
   using MF = Mfma<T>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
   constexpr int MI = Cfg::MI, KI = Cfg::KI, TM = Cfg::TM, TN = Cfg::TN;
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi
   // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each XCD one
   // contiguous range of tiles so that neighbouring tiles share its L2.
   const int chunk = (p.num_tiles + 7) >> 3;
-  const int t = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+  const int t = (wg & 7) * chunk + (wg >> 3);
   if (t >= p.num_tiles) return;
 
   int tm, tn;
@@ -225,7 +225,6 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi
     tn = r / rows;
   }
   const int m0 = tm * BM, n0 = tn * BN;
-  const int z = blockIdx.y;
   const int kbeg = z * p.k_chunk;
   const int kend = min(p.K, kbeg + p.k_chunk);
 
@@ -298,6 +297,44 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi
   }
 }
 
+template <typename T, class Cfg, class Epi>
+__global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi) {
+  gemm_tile_body<T, Cfg, Epi>(p, epi, blockIdx.x, blockIdx.y);
+}
+
+// One problem per blockIdx.z, described in device memory (sizes may be produced by earlier
+// kernels of the same stream); workgroups beyond a problem's tile count return at once.
+template <typename T>
+struct BatchedGemm {
+  GemmProblem<T> p;
+  EpiStore<T> e;
+};
+template <typename T, class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void gemm_batched_kernel(const BatchedGemm<T>* __restrict__ batch) {
+  const BatchedGemm<T> b = batch[blockIdx.z];
+  if (b.p.M <= 0 || b.p.N <= 0) return;
+  gemm_tile_body<T, Cfg, EpiStore<T>>(b.p, b.e, blockIdx.x, 0);
+}
+
+// Device-side twin of make_problem for the default tile.
+template <typename T, class Cfg>
+__device__ __forceinline__ void fill_batched(BatchedGemm<T>& b, int transA, int transB, int M, int N, int K,
+                                             const T* A, int64_t lda, const T* B, int64_t ldb, T* C, int64_t ldc,
+                                             T alpha, T beta) {
+  constexpr int VW = Vec16<T>::W;
+  b.p.A = A; b.p.B = B; b.p.lda = lda; b.p.ldb = ldb;
+  b.p.M = M; b.p.N = N; b.p.K = K;
+  b.p.transA = transA; b.p.transB = transB;
+  b.p.vecA = ((uintptr_t)A % 16 == 0) && (lda % VW == 0) && ((transA ? K : M) % VW == 0);
+  b.p.vecB = ((uintptr_t)B % 16 == 0) && (ldb % VW == 0) && ((transB ? N : K) % VW == 0);
+  b.p.tiles_m = (M + Cfg::BM - 1) / Cfg::BM;
+  b.p.tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
+  b.p.num_tiles = b.p.tiles_m * b.p.tiles_n;
+  b.p.lower = 0;
+  b.p.k_chunk = ((K > 0 ? K : 1) + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
+  b.e.C = C; b.e.ldc = ldc; b.e.alpha = alpha; b.e.beta = beta;
+}
+
 // Sum split-K partials and apply alpha/beta.
 template <typename T>
 __global__ void reduce_partials_kernel(const T* __restrict__ part, int splits, int64_t slab, int M, int N, T* C,
@@ -325,16 +362,27 @@ struct DefaultTile<double> {
   using type = GemmTile<double, 128, 128, 8, 2, 2>;
 };
 
+// Tile for products whose M extent is a panel width (32): tall-skinny block-reflector work.
+template <typename T>
+struct SkinnyTile;
+template <>
+struct SkinnyTile<float> {
+  using type = GemmTile<float, 32, 128, 32, 1, 4>;
+};
+template <>
+struct SkinnyTile<double> {
+  using type = GemmTile<double, 32, 128, 16, 1, 4>;
+};
+
 template <typename T>
 static inline bool vec_ok(const T* p, int64_t ld, int contig_extent) {
   constexpr int VW = Vec16<T>::W;
   return (reinterpret_cast<uintptr_t>(p) % 16 == 0) && (ld % VW == 0) && (contig_extent % VW == 0);
 }
 
-template <typename T>
+template <typename T, class Cfg = typename DefaultTile<T>::type>
 static inline GemmProblem<T> make_problem(int transA, int transB, int M, int N, int K, const T* A, int64_t lda,
                                           const T* B, int64_t ldb, bool lower) {
-  using Cfg = typename DefaultTile<T>::type;
   GemmProblem<T> p;
   p.A = A; p.B = B; p.lda = lda; p.ldb = ldb;
   p.M = M; p.N = N; p.K = K;
@@ -350,9 +398,8 @@ static inline GemmProblem<T> make_problem(int transA, int transB, int M, int N, 
   return p;
 }
 
-template <typename T, class Epi>
+template <typename T, class Epi, class Cfg = typename DefaultTile<T>::type>
 static inline int launch_gemm(hipStream_t stream, const GemmProblem<T>& p, const Epi& epi, int k_splits = 1) {
-  using Cfg = typename DefaultTile<T>::type;
   if (p.M <= 0 || p.N <= 0) return kOk;
   const int chunk = (p.num_tiles + 7) / 8;
   dim3 grid(8 * chunk, k_splits, 1);
@@ -364,19 +411,18 @@ static inline int launch_gemm(hipStream_t stream, const GemmProblem<T>& p, const
 // C = alpha*op(A)*op(B) + beta*C.  If `partials` is non-null and k_splits > 1 the K range is
 // cut into k_splits slices whose partial products are summed by a second kernel (fixed
 // order, so the result does not depend on scheduling).
-template <typename T>
+template <typename T, class Cfg = typename DefaultTile<T>::type>
 static inline int gemm(hipStream_t stream, int transA, int transB, int M, int N, int K, T alpha, const T* A,
                        int64_t lda, const T* B, int64_t ldb, T beta, T* C, int64_t ldc, int k_splits = 1,
                        T* partials = nullptr) {
-  using Cfg = typename DefaultTile<T>::type;
   if (M <= 0 || N <= 0) return kOk;
-  GemmProblem<T> p = make_problem<T>(transA, transB, M, N, K, A, lda, B, ldb, false);
+  GemmProblem<T> p = make_problem<T, Cfg>(transA, transB, M, N, K, A, lda, B, ldb, false);
   if (k_splits > 1 && partials != nullptr && K > Cfg::BK) {
     int64_t slabs = ceil_div64(K, Cfg::BK);
     p.k_chunk = (int)(ceil_div64(slabs, k_splits) * Cfg::BK);
     int splits = (int)ceil_div64(K, p.k_chunk);
     EpiPartial<T> ep{partials, (int64_t)M, (int64_t)M * N};
-    int rc = launch_gemm<T>(stream, p, ep, splits);
+    int rc = launch_gemm<T, EpiPartial<T>, Cfg>(stream, p, ep, splits);
     if (rc) return rc;
     int64_t total = (int64_t)M * N;
     hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3((unsigned)ceil_div64(total, 256)), dim3(256), 0, stream,
@@ -385,7 +431,7 @@ static inline int gemm(hipStream_t stream, int transA, int transB, int M, int N,
     return kOk;
   }
   EpiStore<T> ep{C, ldc, alpha, beta};
-  return launch_gemm<T>(stream, p, ep, 1);
+  return launch_gemm<T, EpiStore<T>, Cfg>(stream, p, ep, 1);
 }
 
 }  // namespace soapmi
