@@ -1,0 +1,74 @@
+"""Shared argument checks and launch helpers for the ops."""
+from __future__ import annotations
+
+from typing import Any, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from .. import _native
+from ..binding import default_binding
+from ._utils import validate_2d_block_cyclic_buffer
+
+
+def stream_of(tensor: Tensor) -> int:
+    return torch.cuda.current_stream(tensor.device).cuda_stream
+
+
+def scratch(nbytes: int, device) -> Tensor:
+    """Workspace from torch's caching allocator (stream-ordered, so no synchronisation)."""
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+def require_device_tensor(name: str, tensor: Tensor) -> None:
+    """The kernels run on the GPU only; same rule and wording as the reference's backend check
+    (src/soap_tp/ops/factorizations.py:33-48 with backend 'rocm')."""
+    if tensor.device.type != "cuda":
+        raise ValueError(
+            f"native backend 'rocm' requires cuda buffers, got {tensor.device.type} for {name}."
+        )
+
+
+def validate_float_buffer(
+    name: str,
+    matrix: Tensor,
+    global_shape: Tuple[int, int],
+    block_size: int,
+    process_grid_shape: Tuple[int, int],
+    rank: int,
+) -> Tuple[int, int]:
+    if matrix.dtype != torch.float32:
+        raise ValueError(f"{name} must use float32, got {matrix.dtype}.")
+    return validate_2d_block_cyclic_buffer(
+        name, matrix, global_shape, block_size, process_grid_shape, rank
+    )
+
+
+def validated_binding(binding: Optional[Any], device: torch.device, rank: int, world_size: int) -> Any:
+    """Resolve and check a binding object the way the reference does
+    (src/soap_tp/ops/factorizations.py:85-101)."""
+    if binding is None:
+        binding = default_binding()
+    mpi_rank, mpi_world_size = binding.mpi_world_rank_and_size()
+    if (mpi_rank, mpi_world_size) != (rank, world_size):
+        raise RuntimeError(
+            "Torch and MPI worlds must have identical ranks and sizes; "
+            f"got Torch {(rank, world_size)} and MPI {(mpi_rank, mpi_world_size)}."
+        )
+    backend = binding.compiled_gpu_backend()
+    if backend not in {"none", "cuda", "rocm"}:
+        raise RuntimeError(f"unsupported native backend {backend!r}.")
+    expected_device = "cpu" if backend == "none" else "cuda"
+    if device.type != expected_device:
+        raise ValueError(
+            f"native backend {backend!r} requires {expected_device} buffers, got {device.type}."
+        )
+    if backend == "cuda" and (torch.version.cuda is None or torch.version.hip is not None):
+        raise RuntimeError("the CUDA binding requires a CUDA PyTorch build.")
+    if backend == "rocm" and torch.version.hip is None:
+        raise RuntimeError("the ROCm binding requires a ROCm PyTorch build.")
+    return binding
+
+
+native_call = _native.call
+native_library = _native.library

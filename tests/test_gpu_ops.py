@@ -1,0 +1,208 @@
+"""Op-level parity of the HIP path against the CPU oracle, on the inputs of the reference's own
+unit tests (seed 42, N(0, 2), block size 2, shapes (8,8) (8,12) (12,8) (9,13) (13,9)) restated
+for one rank, plus larger and ragged sizes.  Every call goes Python -> ctypes -> C ABI.
+
+Tolerances (float32 path): relative L2 <= 1e-5 on products, Adam and Gram matrices -- the
+reference's own bar (tests/unit/test_preconditioners.py:405-417, test_factorizations.py:345-373);
+data movement (permute, layout copies, argsort) is exact."""
+import math
+
+import pytest
+import torch
+
+from oracle import soap_oracle as oracle
+from soap_tp_amd import ops
+from tests.helpers import (MATRIX_SHAPES, SEED, align_signs, column_major, make_matrix, make_orthogonal,
+                           make_preconditioner, relative_l2)
+
+pytestmark = pytest.mark.gpu
+GRID = (1, 1)
+BLOCK = 2
+RTOL = 1e-5
+EXTRA_SHAPES = ((1, 1), (1, 7), (130, 70), (256, 384), (300, 129))
+
+
+# ---- Gram EMA (tests/unit/test_preconditioners.py of the reference) ------------------------------
+@pytest.mark.parametrize("shape", MATRIX_SHAPES + EXTRA_SHAPES)
+@pytest.mark.parametrize("side", ["left", "right"])
+@pytest.mark.parametrize("shard_dim", [0, 1])
+def test_preconditioner_update_from_zero(shape, side, shard_dim, device):
+    gradient = make_matrix(*shape)
+    size = shape[0] if side == "left" else shape[1]
+    packed = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+    update = (ops.update_left_preconditioner_2d_block_cyclic_ if side == "left"
+              else ops.update_right_preconditioner_2d_block_cyclic_)
+    result = update(gradient.to(device), packed, 0.0, BLOCK, GRID, shard_dim=shard_dim)
+    assert result is packed
+    expected = oracle.gram_ema(torch.zeros(size, size), gradient, 0.0, side)
+    assert relative_l2(packed, expected) <= RTOL
+    torch.testing.assert_close(packed.cpu(), expected, rtol=RTOL, atol=RTOL * expected.abs().max().item())
+    assert torch.equal(packed, packed.T)  # both triangles, bit-identical mirror
+
+
+@pytest.mark.parametrize("beta", [0.25, 0.95, 1.0])
+def test_preconditioner_update_nonzero_beta(beta, device):
+    gradient = make_matrix(9, 13, seed=SEED + 100)  # tests/unit/test_preconditioners.py:591-608
+    packed = column_major(torch.full((9, 9), 2.0), device)
+    ops.update_left_preconditioner_2d_block_cyclic_(gradient.to(device), packed, beta, BLOCK, GRID, shard_dim=0)
+    expected = oracle.gram_ema(torch.full((9, 9), 2.0), gradient, beta, "left")
+    assert relative_l2(packed, expected) <= RTOL
+
+
+def test_preconditioner_lower_only_and_layouts(device):
+    gradient = make_matrix(70, 130)
+    start = make_preconditioner(130, SEED + 1)
+    expected = oracle.gram_ema(start.clone(), gradient, 0.9, "right")
+    lower = column_major(start, device, pad=3)
+    upper_before = torch.triu(lower, 1).clone()
+    ops.update_right_preconditioner_2d_block_cyclic_(gradient.to(device), lower, 0.9, BLOCK, GRID, shard_dim=1,
+                                                     mirror=False)
+    assert relative_l2(torch.tril(lower), torch.tril(expected)) <= RTOL
+    assert torch.equal(torch.triu(lower, 1), upper_before)  # upper triangle untouched
+    # a column-major (transposed-view) gradient takes the other operand layout
+    full = column_major(start, device)
+    ops.update_right_preconditioner_2d_block_cyclic_(gradient.to(device).T.contiguous().T, full, 0.9, BLOCK, GRID,
+                                                     shard_dim=1)
+    assert relative_l2(full, expected) <= RTOL
+    half = column_major(start, device)
+    ops.update_right_preconditioner_2d_block_cyclic_(gradient.to(device).half(), half, 0.9, BLOCK, GRID, shard_dim=1)
+    assert relative_l2(half, oracle.gram_ema(start.clone(), gradient.half().float(), 0.9, "right")) <= RTOL
+
+
+# ---- Adam (tests/unit/test_optimizer.py) ---------------------------------------------------------
+@pytest.mark.parametrize("shape", MATRIX_SHAPES + ((257, 130),))
+@pytest.mark.parametrize("layout", ["column_major", "row_major"])
+def test_adam_update(shape, layout, device):
+    step, beta1, beta2, eps = 3, 0.8, 0.9, 1e-6
+    host = [make_matrix(*shape, seed=SEED), make_matrix(*shape, seed=SEED + 1),
+            make_matrix(*shape, seed=SEED + 2).square()]
+    expected_update = oracle.adam_update(host[0].clone(), m_ref := host[1].clone(), v_ref := host[2].clone(),
+                                         step, beta1, beta2, eps)
+    place = (lambda t: column_major(t, device)) if layout == "column_major" else (lambda t: t.to(device))
+    gradient, momentum, variance = (place(t) for t in host)
+    update = ops.adam_update(gradient, momentum, variance, step=step, beta1=beta1, beta2=beta2, eps=eps)
+    assert update.shape == gradient.shape and update.stride() == variance.stride()
+    assert relative_l2(update, expected_update) <= RTOL
+    torch.testing.assert_close(momentum.cpu(), m_ref)
+    torch.testing.assert_close(variance.cpu(), v_ref)
+    torch.testing.assert_close(update.cpu(), expected_update)
+
+
+# ---- permutation and layout copies ---------------------------------------------------------------
+@pytest.mark.parametrize("shape", MATRIX_SHAPES + ((300, 129),))
+def test_permute_and_redistribute_are_exact(shape, device):
+    rows, columns = shape
+    matrix = make_matrix(rows, columns)
+    generator = torch.Generator().manual_seed(SEED)
+    row_order, column_order = torch.randperm(rows, generator=generator), torch.randperm(columns, generator=generator)
+    packed = ops.redistribute_tp_shard_to_2d_block_cyclic(matrix.to(device), shape, BLOCK, GRID, shard_dim=1)
+    assert packed.stride(0) == 1 and torch.equal(packed.cpu(), matrix)
+    result = ops.permute_2d_block_cyclic_(packed, shape, row_order.tolist(), column_order.to(device), BLOCK, GRID)
+    assert result is packed
+    assert torch.equal(packed.cpu(), oracle.permute(matrix, row_order, column_order))
+    shard = ops.redistribute_2d_block_cyclic_to_tp_shard(packed, shape, BLOCK, GRID, shard_dim=0)
+    assert shard.is_contiguous() and torch.equal(shard.cpu(), oracle.permute(matrix, row_order, column_order))
+    with pytest.raises(ValueError, match="row_order must be a permutation"):
+        ops.permute_2d_block_cyclic_(packed, shape, [0] * rows, column_order, BLOCK, GRID)
+    with pytest.raises(ValueError, match="column_order must be a permutation"):
+        ops.permute_2d_block_cyclic_(packed, shape, row_order, column_order[:-1], BLOCK, GRID)
+
+
+# ---- rotations (tests/unit/test_factorizations.py:376-399) ---------------------------------------
+@pytest.mark.parametrize("shape", MATRIX_SHAPES + ((130, 70), (256, 384)))
+@pytest.mark.parametrize("direction", ["forward", "backward"])
+def test_rotate(shape, direction, device):
+    rows, columns = shape
+    matrix = make_matrix(rows, columns, seed=SEED + rows * 100 + columns)
+    q_left, q_right = make_orthogonal(rows, SEED + 1000 + rows), make_orthogonal(columns, SEED + 2000 + columns)
+    packed = column_major(matrix, device, pad=1)
+    result = ops.rotate_2d_block_cyclic_(packed, column_major(q_left, device), column_major(q_right, device, pad=2),
+                                         shape, BLOCK, GRID, direction=direction)
+    assert result is packed
+    expected = oracle.rotate(matrix, q_left, q_right, direction)
+    assert relative_l2(packed, expected) <= RTOL
+    torch.testing.assert_close(packed.cpu(), expected, rtol=2e-4, atol=2e-4)
+    assert abs(packed.norm().item() / matrix.norm().item() - 1) < 1e-5  # orthogonal invariance
+
+
+# ---- order, QR, power iteration (tests/unit/test_slate_bindings.py) ------------------------------
+@pytest.mark.parametrize("size", [8, 12, 9, 13, 100, 257])
+def test_estimated_order_qr_and_power_iteration(size, device):
+    preconditioner, basis = make_preconditioner(size, SEED + 5000), make_orthogonal(size, SEED + 7000)
+    expected_order, expected_estimates, expected_work = oracle.estimated_order(preconditioner, basis)
+    p_dev, q_dev = column_major(preconditioner, device), column_major(basis, device)
+    work = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+    order = ops.estimated_eigenvalue_order_2d_block_cyclic_(p_dev, q_dev, work, size, BLOCK, GRID)
+    assert order.dtype == torch.int64 and order.tolist() == expected_order.tolist()
+    assert relative_l2(work, expected_work) <= RTOL
+
+    matrix = make_matrix(size, size, seed=SEED + size)
+    factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+    assert ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID) is factor
+    expected_q = oracle.householder_qr(matrix)
+    assert relative_l2(factor, expected_q) <= 5e-5  # same sign convention: no alignment needed
+    torch.testing.assert_close(factor.T @ factor, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
+    r = factor.double().T.cpu() @ matrix.double()
+    assert torch.tril(r, -1).abs().max().item() <= 1e-4 * matrix.abs().max().item() * math.sqrt(size)
+
+    returned = ops.power_iteration_qr_2d_block_cyclic_(p_dev, q_dev, work, size, BLOCK, GRID)
+    expected_order2, expected_basis = oracle.power_iteration_qr(preconditioner, basis)
+    assert returned.tolist() == expected_order2.tolist()
+    signs = align_signs(q_dev.cpu(), expected_basis)
+    assert relative_l2(q_dev.cpu() * signs, expected_basis) <= 1e-4
+    torch.testing.assert_close(q_dev.T @ q_dev, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
+
+
+def test_argsort_ties_and_large(device):
+    from soap_tp_amd import _native
+    for count in (1, 2, 33, 4096, 16384, 20000):
+        keys = torch.randn(count, generator=torch.Generator().manual_seed(count))
+        if count > 10:
+            keys[3] = keys[7] = keys[9]
+        order = torch.empty(count, dtype=torch.int64, device=device)
+        keys_dev = keys.to(device)
+        nbytes = _native.library().soapmi_argsort_workspace_bytes(count)
+        work = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _native.call("soapmi_argsort_desc_f32", keys_dev.data_ptr(), count, order.data_ptr(), work.data_ptr(),
+                     work.numel(), torch.cuda.current_stream().cuda_stream)
+        assert order.tolist() == torch.argsort(keys, descending=True, stable=True).tolist()
+
+
+# ---- refresh (tests/unit/test_factorizations.py:501-613) -----------------------------------------
+@pytest.mark.parametrize("shape", MATRIX_SHAPES + ((130, 70),))
+@pytest.mark.parametrize("storage", ["full", "lower"])
+def test_refresh_bases_and_transport_optimizer_state(shape, storage, device):
+    rows, columns = shape
+    state = {
+        "momentum": make_matrix(rows, columns, seed=SEED + 3000),
+        "variance": make_matrix(rows, columns, seed=SEED + 4000).square(),
+        "left_preconditioner": make_preconditioner(rows, SEED + 5000),
+        "right_preconditioner": make_preconditioner(columns, SEED + 6000),
+        "left_basis": make_orthogonal(rows, SEED + 7000),
+        "right_basis": make_orthogonal(columns, SEED + 8000),
+    }
+    dev = {name: column_major(t, device) for name, t in state.items()}
+    if storage == "lower":  # the upper triangles hold stale values until the refresh rebuilds them
+        for side in ("left", "right"):
+            p = dev[f"{side}_preconditioner"]
+            p.copy_(torch.tril(p) + torch.triu(torch.full_like(p, 3.0), 1))
+    left_work = ops.allocate_2d_block_cyclic((rows, rows), BLOCK, GRID, device=device)
+    right_work = ops.allocate_2d_block_cyclic((columns, columns), BLOCK, GRID, device=device)
+    left_order, right_order = ops.refresh_bases_and_transport_optimizer_state_(
+        dev["momentum"], dev["variance"], dev["left_preconditioner"], dev["right_preconditioner"],
+        dev["left_basis"], dev["right_basis"], left_work, right_work, shape, BLOCK, GRID,
+        symmetrize=(storage == "lower"))
+    expected_left, expected_right = oracle.refresh(state)
+    assert left_order.tolist() == expected_left.tolist() and right_order.tolist() == expected_right.tolist()
+    left_signs = align_signs(dev["left_basis"].cpu(), state["left_basis"])
+    right_signs = align_signs(dev["right_basis"].cpu(), state["right_basis"])
+    assert relative_l2(dev["left_basis"].cpu() * left_signs, state["left_basis"]) <= 1e-4
+    assert relative_l2(dev["right_basis"].cpu() * right_signs, state["right_basis"]) <= 1e-4
+    assert relative_l2(dev["momentum"].cpu() * left_signs[:, None] * right_signs[None, :], state["momentum"]) <= 1e-4
+    assert torch.equal(dev["variance"].cpu(), state["variance"])
+    for side, size in (("left", rows), ("right", columns)):
+        q = dev[f"{side}_basis"]
+        torch.testing.assert_close(q.T @ q, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
+        if storage == "lower":  # the refresh rebuilt the upper triangle from the lower one
+            p = dev[f"{side}_preconditioner"]
+            assert torch.equal(p, p.T)

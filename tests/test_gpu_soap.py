@@ -1,0 +1,280 @@
+"""End-to-end parity of ``soap_step`` on the GPU against the CPU oracle and the golden trajectory
+of the original optimizer, restating tests/unit/test_soap.py of the reference for one rank
+(10 iterations, refresh every 2, betas 0.75 / 0.8 / 0.9, eps 1e-6, N(0, 2) gradients, block 2),
+then BASELINE's first configuration and size-independent properties at the benchmark sizes.
+
+Bar: relative Frobenius error <= 1e-4 on updates, moments and Gram matrices (float32 path).
+Where eigenvectors are not determined to working precision by the data (clusters of nearly equal
+eigenvalues, the zero eigenspace of a rectangular gradient's Gram matrix) the comparison is made
+conditionally on the bases: the GPU's bases and sort orders are handed to the oracle, which then
+has to reproduce update, moments and Gram matrices; the bases themselves are checked by
+invariants (residual, orthogonality, eigenvalues, subspaces of separated clusters)."""
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import soap_tp_amd
+from oracle import soap_oracle as oracle
+from soap_tp_amd import soap as soap_module
+from soap_tp_amd.binding import NativeBinding
+from tests.helpers import SEED, relative_l2, subspace_distance
+
+pytestmark = pytest.mark.gpu
+GRID = (1, 1)
+GOLDEN = Path(__file__).resolve().parent / "golden" / "soap_trajectory.npz"
+CONFIG = dict(preconditioner_beta=0.75, beta1=0.8, beta2=0.9, eps=1e-6, basis_refresh_interval=2)
+TOL = 1e-4
+
+
+def _reference_gradients(shape, iterations=10):
+    generator = torch.Generator().manual_seed(SEED + 1)
+    return [torch.normal(0, 2, size=shape, generator=generator) for _ in range(iterations)]
+
+
+def _run_gpu(gradients, device, shard_dim=1, block_size=2, record=None, monkeypatch=None, **kwargs):
+    """Run soap_step over ``gradients``; with ``record`` (a dict) and monkeypatch, store the bases
+    after initialisation / each refresh and the refresh orders, keyed by step."""
+    if record is not None:
+        original = soap_module.refresh_bases_and_transport_optimizer_state_
+
+        def recording(*args, **kw):
+            orders = original(*args, **kw)
+            record["orders"] = tuple(o.cpu() for o in orders)
+            return orders
+
+        monkeypatch.setattr(soap_module, "refresh_bases_and_transport_optimizer_state_", recording)
+    state, updates = {}, []
+    shape = tuple(gradients[0].shape)
+    for gradient in gradients:
+        if record is not None:
+            record.pop("orders", None)
+        update = soap_tp_amd.soap_step(gradient.to(device), state, global_shape=shape, shard_dim=shard_dim,
+                                       block_size=block_size, process_grid_shape=GRID, **kwargs)
+        updates.append(update.cpu())
+        if record is not None:
+            step = int(state["step"])
+            if step == 0 or "orders" in record:
+                entry = (state["left_basis"].cpu().clone(), state["right_basis"].cpu().clone())
+                if "orders" in record:
+                    entry = entry + record["orders"]
+                record.setdefault("bases", {})[step] = entry
+    return updates, state
+
+
+def _run_oracle(gradients, bases_override=None, **kwargs):
+    state, updates = {}, []
+    for gradient in gradients:
+        updates.append(oracle.soap_step(gradient, state, bases_override=bases_override, **kwargs))
+    return updates, state
+
+
+def _assert_match_except_sign_flips(actual, reference, bases, allowed_fraction=0.01):
+    """Compare in the eigenbasis coordinates, where a flipped sign stays in one entry."""
+    q_left, q_right = (q.double() for q in bases)
+    actual = q_left.T @ actual.double() @ q_right
+    reference = q_left.T @ reference.double() @ q_right
+    difference = (actual - reference).abs()
+    outliers = difference > 1e-3 * reference.abs().max().item()
+    assert outliers.sum().item() <= max(1, int(allowed_fraction * reference.numel()))
+    kept = ~outliers
+    assert relative_l2(actual[kept], reference[kept]) <= 10 * TOL
+
+
+def _full(matrix):
+    matrix = matrix.cpu()
+    return torch.tril(matrix) + torch.tril(matrix, -1).T
+
+
+# ---- the reference's end-to-end comparison -------------------------------------------------------
+@pytest.mark.parametrize("shape,implementation", [((8, 8), "elpa"), ((12, 12), "elpa"), ((8, 8), "eigh"),
+                                                  ((12, 12), "eigh"), ((20, 20), "eigh")])
+@pytest.mark.parametrize("shard_dim", [0, 1])
+def test_soap_step_matches_oracle_and_golden_trajectory(shape, implementation, shard_dim, device):
+    gradients = _reference_gradients(shape)
+    updates, state = _run_gpu(gradients, device, shard_dim=shard_dim, basis_implementation=implementation, **CONFIG)
+    expected, expected_state = _run_oracle(gradients, basis_implementation=implementation, **CONFIG)
+    golden = np.load(GOLDEN)[f"updates_{shape[0]}x{shape[1]}"]
+    first = gradients[0]
+    initial_bases = tuple(
+        oracle.eigh_descending(oracle.gram_ema(torch.zeros(n, n), first, CONFIG["preconditioner_beta"], side),
+                               implementation)[1]
+        for side, n in (("left", shape[0]), ("right", shape[1])))
+    assert torch.count_nonzero(updates[0]) == 0  # warm-up call returns exact zeros (test_soap.py:791-801)
+    assert updates[0].dtype == torch.float32 and updates[0].shape == shape
+    for iteration in range(1, len(gradients)):
+        # On the first real step both moments are built from one sample, so the update is
+        # g / (|g| + eps'): a sign function, whose response to a float32-level change of a
+        # near-zero rotated-gradient entry is O(1) in that entry.  One such entry out of 400 is
+        # what (20, 20) shows there; every later step, and the same step conditionally on the
+        # bases (next test), meets the 1e-4 bar.
+        # The golden file shows it too: made on another CPU, it differs from the same oracle run
+        # on this host in exactly such an entry.  So on that step up to 1 % of the entries may
+        # disagree; the others must meet the bar like every other step.
+        for reference in (expected[iteration], torch.from_numpy(golden[iteration])):
+            if iteration == 1:
+                _assert_match_except_sign_flips(updates[iteration], reference, initial_bases)
+            else:
+                # a flipped entry of step 1 stays in the moments and decays with beta1 = 0.8
+                tolerance = 1e-3 if shape == (20, 20) else TOL
+                assert relative_l2(updates[iteration], reference) <= tolerance, f"iteration {iteration}"
+    assert state["step"] == len(gradients) - 1 == expected_state["step"]
+    assert relative_l2(_full(state["left_preconditioner"]), expected_state["left_preconditioner"]) <= TOL
+    assert relative_l2(_full(state["right_preconditioner"]), expected_state["right_preconditioner"]) <= TOL
+    assert sorted(state) == sorted(list(soap_module.STATE_BUFFERS) + ["step"])
+    for name in soap_module.STATE_BUFFERS:
+        assert state[name].stride(0) == 1 and state[name].dtype == torch.float32
+
+
+@pytest.mark.parametrize("shape", [(8, 8), (20, 20), (12, 20), (20, 12), (9, 13)])
+@pytest.mark.parametrize("implementation", ["elpa", "eigh"])
+def test_soap_step_conditional_on_bases(shape, implementation, device, monkeypatch):
+    gradients = _reference_gradients(shape)
+    record = {}
+    updates, state = _run_gpu(gradients, device, record=record, monkeypatch=monkeypatch,
+                              basis_implementation=implementation, **CONFIG)
+    assert sorted(record["bases"]) == [0, 2, 4, 6, 8]
+    expected, expected_state = _run_oracle(gradients, bases_override=record["bases"],
+                                           basis_implementation=implementation, **CONFIG)
+    for iteration in range(len(gradients)):
+        assert relative_l2(updates[iteration], expected[iteration]) <= TOL, f"iteration {iteration}"
+    for name in ("momentum", "variance"):
+        assert relative_l2(state[name], expected_state[name]) <= TOL, name
+    for side in ("left", "right"):
+        assert relative_l2(_full(state[f"{side}_preconditioner"]), expected_state[f"{side}_preconditioner"]) <= TOL
+        q = state[f"{side}_basis"]
+        torch.testing.assert_close(q.T @ q, torch.eye(q.shape[0], device=q.device), rtol=1e-4, atol=1e-4)
+
+
+class _CountingSlateBinding:
+    """Delegating proxy, as in tests/unit/test_soap.py:402-412 of the reference."""
+
+    def __init__(self, binding):
+        self._binding = binding
+        self.qr_calls = 0
+        self.rotations = 0
+
+    def __getattr__(self, name):
+        return getattr(self._binding, name)
+
+    def slate_qr_float(self, *args, **kwargs):
+        self.qr_calls += 1
+        return self._binding.slate_qr_float(*args, **kwargs)
+
+    def slate_forward_rotation_float(self, *args, **kwargs):
+        self.rotations += 1
+        return self._binding.slate_forward_rotation_float(*args, **kwargs)
+
+
+@pytest.mark.parametrize("shape", [(12, 12), (13, 9)])
+def test_injected_bindings_see_reference_call_counts_and_match_fused_path(shape, device):
+    gradients = _reference_gradients(shape)
+    counted = _CountingSlateBinding(NativeBinding())
+    via_binding, state_b = _run_gpu(gradients, device, slate_binding=counted, elpa_binding=NativeBinding(), **CONFIG)
+    fused, state_f = _run_gpu(gradients, device, **CONFIG)
+    steps = len(gradients) - 1
+    refreshes = steps // CONFIG["basis_refresh_interval"]
+    assert (state_b["step"], counted.qr_calls) == (steps, 2 * refreshes)  # test_soap.py:844-849
+    assert counted.rotations == steps + refreshes
+    for iteration in range(len(gradients)):
+        assert relative_l2(via_binding[iteration], fused[iteration]) <= 2e-5, f"iteration {iteration}"
+    full, state_full = _run_gpu(gradients, device, preconditioner_storage="full", **CONFIG)
+    for iteration in range(len(gradients)):
+        assert torch.equal(full[iteration], fused[iteration])
+    p = state_full["left_preconditioner"]
+    assert torch.equal(p, p.T)
+
+
+def test_profile_lines(device, monkeypatch, capsys):
+    import json
+
+    monkeypatch.setenv("SOAP_PROFILE", "1")
+    monkeypatch.setenv("SOAP_PROFILE_STEPS", "0,2")
+    _run_gpu(_reference_gradients((8, 8), 3), device, **CONFIG)
+    lines = [line for line in capsys.readouterr().out.splitlines() if line.startswith("SOAP_PROFILE ")]
+    records = [json.loads(line[len("SOAP_PROFILE "):]) for line in lines]
+    assert {r["step"] for r in records} == {0, 2}
+    stages = {r["stage"] for r in records if r["step"] == 2}
+    assert {"gradient", "projected_gradient", "momentum_after_adam", "variance_after_adam", "coordinate_update",
+            "backrotated_update", "returned_update", "left_preconditioner_after_step", "left_basis_after_step",
+            "momentum_after_step", "variance_after_step"} <= stages
+    first = records[0]
+    assert first["impl"] == "tp" and first["shape"] == [8, 8] and len(first["values"]) == 64
+
+
+# ---- BASELINE configuration 1: 1024 x 1024, rank 32 low-rank-plus-noise, 20 steps, refresh 10 ----
+def test_baseline_config_1024(device, monkeypatch):
+    rows = columns = 1024
+    kwargs = dict(preconditioner_beta=0.95, beta1=0.95, beta2=0.95, eps=1e-8, basis_refresh_interval=10)
+    gradients = [oracle.low_rank_plus_noise(rows, columns, 32, seed=SEED + t) for t in range(20)]
+    record = {}
+    updates, state = _run_gpu(gradients, device, block_size=128, record=record, monkeypatch=monkeypatch, **kwargs)
+    assert sorted(record["bases"]) == [0, 10]
+    expected, expected_state = _run_oracle(gradients, bases_override=record["bases"], **kwargs)
+    worst = max(relative_l2(updates[t], expected[t]) for t in range(1, 20))
+    assert worst <= TOL, worst
+    for name in ("momentum", "variance"):
+        assert relative_l2(state[name], expected_state[name]) <= TOL, name
+    for side in ("left", "right"):
+        assert relative_l2(_full(state[f"{side}_preconditioner"]), expected_state[f"{side}_preconditioner"]) <= TOL
+    # bases: invariants against the oracle's own (unconditioned) initialisation
+    first = gradients[0]
+    gram = 0.05 * first @ first.T
+    values, vectors = oracle.eigh_descending(gram, "elpa")
+    q0 = record["bases"][0][0]
+    rayleigh = torch.diagonal(q0.double().T @ gram.double() @ q0.double())
+    assert (rayleigh - values.double()).abs().max().item() <= 1e-5 * values[0].item()
+    assert subspace_distance(q0[:, :32], vectors[:, :32]) <= 1e-3           # the rank-32 signal subspace
+    torch.testing.assert_close(q0.T @ q0, torch.eye(rows), rtol=1e-4, atol=1e-4)
+    residual = gram.double() @ q0.double() - q0.double() * rayleigh
+    assert torch.linalg.matrix_norm(residual).item() <= 1e-5 * torch.linalg.matrix_norm(gram.double()).item()
+    q10 = record["bases"][10][0]
+    torch.testing.assert_close(q10.T @ q10, torch.eye(rows), rtol=1e-4, atol=1e-4)
+    left_order = record["bases"][10][2]
+    assert sorted(left_order.tolist()) == list(range(rows))
+
+
+# ---- size-independent properties at the benchmark sizes -------------------------------------------
+@pytest.mark.parametrize("shape,rank", [((4096, 4096), 64), ((4096, 11008), 128)])
+def test_properties_at_benchmark_sizes(shape, rank, device):
+    rows, columns = shape
+    beta = 0.95
+    kwargs = dict(global_shape=shape, shard_dim=1, block_size=128, process_grid_shape=GRID,
+                  basis_refresh_interval=2, basis_implementation="elpa")
+    state = {}
+    norms, traces = [], []
+    for t in range(3):  # warm-up/initialisation, one plain step, one refresh step
+        gradient = oracle.low_rank_plus_noise(rows, columns, rank, seed=SEED + t).to(device)
+        update = soap_tp_amd.soap_step(gradient, state, **kwargs)
+        norms.append(gradient.double().norm().item() ** 2)
+        traces.append((torch.diagonal(state["left_preconditioner"]).double().sum().item(),
+                       torch.diagonal(state["right_preconditioner"]).double().sum().item()))
+        if t == 0:
+            assert torch.count_nonzero(update) == 0
+        else:
+            assert torch.isfinite(update).all()
+    # trace(P_t) = beta trace(P_{t-1}) + (1 - beta) ||G_t||_F^2 for both Gram matrices
+    for side in (0, 1):
+        expected = 0.0
+        for t in range(3):
+            expected = beta * expected + (1 - beta) * norms[t]
+            assert abs(traces[t][side] - expected) <= 1e-4 * expected
+    for name, size in (("left_basis", rows), ("right_basis", columns)):
+        q = state[name]
+        gram = q.T @ q
+        assert (gram - torch.eye(size, device=device)).abs().max().item() <= 1e-4
+    for side in ("left", "right"):
+        p = state[f"{side}_preconditioner"]
+        assert torch.equal(p, p.T)  # the refresh rebuilt the upper triangle from the lower one
+    # an explicit refresh permutes variance (same multiset of values) and moves momentum between
+    # orthonormal bases (same Frobenius norm)
+    variance_sorted = torch.sort(state["variance"].flatten()).values.clone()
+    momentum_norm = state["momentum"].double().norm().item()
+    left_order, right_order = soap_tp_amd.ops.refresh_bases_and_transport_optimizer_state_(
+        state["momentum"], state["variance"], state["left_preconditioner"], state["right_preconditioner"],
+        state["left_basis"], state["right_basis"], state["left_work"], state["right_work"], shape, 128, GRID)
+    assert torch.equal(torch.sort(state["variance"].flatten()).values, variance_sorted)
+    assert abs(state["momentum"].double().norm().item() / momentum_norm - 1) <= 1e-4
+    assert torch.equal(torch.sort(left_order).values, torch.arange(rows, device=device))
+    assert torch.equal(torch.sort(right_order).values, torch.arange(columns, device=device))
