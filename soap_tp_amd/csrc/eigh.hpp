@@ -19,7 +19,8 @@ struct EighWorkspace {
   T* tau;
   TrdWorkspace<T> trd;
   DcWorkspace<T> dc;
-  QrWorkspace<T> br;  // block-reflector scratch for the back-transformation
+  BlockReflectorWs<T> br;  // block-reflector scratch for the back-transformation
+  T* t_block;              // kBrMax x kBrMax
 };
 
 template <typename T, class WS>
@@ -30,7 +31,8 @@ static inline void eigh_workspace_layout(WS& ws, int64_t n, EighWorkspace<T>* ou
   w.tau = ws.template take<T>(n);
   trd_workspace_layout<T>(ws, n, out ? &w.trd : nullptr);
   dc_workspace_layout<T>(ws, n, out ? &w.dc : nullptr);
-  qr_workspace_layout<T>(ws, n, out ? &w.br : nullptr);
+  block_reflector_layout<T>(ws, n, out ? &w.br : nullptr);
+  w.t_block = ws.template take<T>(kBrMax * kBrMax);
   if (out) *out = w;
 }
 
@@ -55,25 +57,20 @@ static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, i
   if (rc) return rc;
   rc = stedc<T>(s, n, ws.d, ws.e, w, Z, ldz, ws.dc);
   if (rc) return rc;
-  // Z <- H_0 H_1 ... H_{n-2} Z, block reflectors applied last panel first.
+  // Z <- H_0 H_1 ... H_{n-2} Z, 128-wide block reflectors applied last block first.
   const int nref = n - 1;  // reflector j lives in column j, rows j+1..n-1
   if (nref <= 0) return kOk;
-  constexpr int NB = kQrNb;
-  const int panels = (int)ceil_div64(nref, NB);
+  constexpr int OB = kBrMax;
+  const int blocks = (int)ceil_div64(nref, OB);
   const int64_t ldv = n;
-  for (int pi = panels - 1; pi >= 0; --pi) {
-    const int p = pi * NB, pe = std::min(nref, p + NB), nbw = pe - p;
+  for (int bi = blocks - 1; bi >= 0; --bi) {
+    const int p = bi * OB, pe = std::min(nref, p + OB), nbw = pe - p;
     const int rows = n - p - 1;
-    hipLaunchKernelGGL((extract_v_kernel<T>), dim3((unsigned)ceil_div64(rows, 256)), dim3(256), 0, s, A, lda, rows, p + 1,
-                       p, nbw, ws.br.vc, ldv);
+    launch_extract_v<T>(s, A, lda, rows, p + 1, p, nbw, ws.br.v, ldv);
     SOAPMI_LAUNCH_CHECK();
-    const int splits = rows >= 2048 ? kQrSplits : 1;
-    rc = gemm<T, typename SkinnyTile<T>::type>(s, 1, 0, nbw, nbw, rows, T(1), ws.br.vc, ldv, ws.br.vc, ldv, T(0),
-                                               ws.br.gram, NB, splits, ws.br.splitk);
+    rc = build_t_factor<T>(s, ws.br, rows, nbw, ldv, ws.tau + p, ws.t_block);
     if (rc) return rc;
-    hipLaunchKernelGGL((larft_kernel<T>), dim3(1), dim3(64), 0, s, ws.br.gram, NB, ws.tau + p, nbw, ws.br.t_all, NB);
-    SOAPMI_LAUNCH_CHECK();
-    rc = apply_block_reflector<T>(s, ws.br, ws.br.t_all, false, rows, nbw, n, ldv, Z + (p + 1), ldz);
+    rc = apply_block_reflector<T>(s, ws.br, ws.t_block, false, rows, nbw, n, ldv, Z + (p + 1), ldz);
     if (rc) return rc;
   }
   return kOk;

@@ -16,19 +16,28 @@ namespace soapmi {
 
 constexpr int kQrNb = 32;
 
+// One butterfly stage: lanes whose bit MASK is set keep the upper HALF values, the others the
+// lower HALF, and each adds what its partner (lane ^ MASK) holds for the same positions.
+template <typename T, int HALF, int MASK>
+__device__ __forceinline__ void butterfly_stage(T (&vals)[32], int lane) {
+  const bool upper = (lane & MASK) != 0;
+#pragma unroll
+  for (int c = 0; c < HALF; ++c) {
+    const T send = upper ? vals[c] : vals[c + HALF];
+    const T keep = upper ? vals[c + HALF] : vals[c];
+    vals[c] = keep + __shfl_xor(send, MASK, 64);
+  }
+}
+
 // After the call lane l holds, in the return value, the sum over the wavefront of vals[(l>>1)&31].
+// Stages are spelled out so that every register index is a compile-time constant.
 template <typename T>
 __device__ __forceinline__ T wave_reduce_32(T (&vals)[32], int lane) {
-#pragma unroll
-  for (int half = 16, mask = 32; half >= 1; half >>= 1, mask >>= 1) {
-    const bool upper = (lane & mask) != 0;
-#pragma unroll
-    for (int c = 0; c < half; ++c) {
-      const T send = upper ? vals[c] : vals[c + half];
-      const T keep = upper ? vals[c + half] : vals[c];
-      vals[c] = keep + __shfl_xor(send, mask, 64);
-    }
-  }
+  butterfly_stage<T, 16, 32>(vals, lane);
+  butterfly_stage<T, 8, 16>(vals, lane);
+  butterfly_stage<T, 4, 8>(vals, lane);
+  butterfly_stage<T, 2, 4>(vals, lane);
+  butterfly_stage<T, 1, 2>(vals, lane);
   return vals[0] + __shfl_xor(vals[0], 1, 64);
 }
 
@@ -38,9 +47,10 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
                                                             const T* __restrict__ piv_in, T* __restrict__ part_out,
                                                             T* __restrict__ piv_out, T* __restrict__ tau, int nwg) {
   constexpr int NB = kQrNb;
-  __shared__ T s_dots[NB];
   __shared__ T s_tc[NB];
   __shared__ T s_wave[4][NB];
+  __shared__ T s_sum8[8][NB];
+  __shared__ T s_piv[NB];
   __shared__ T s_scal[3];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = p + blockIdx.x * 256 + tid;
@@ -54,15 +64,30 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
   for (int c = 0; c < NB; ++c) a[c] = (live && c < ncol) ? A[r + (int64_t)(c0 + c) * lda] : T(0);
 
   if (apply) {
-    if (tid < ncol) {
+    {
+      // fixed-order sum of the per-workgroup partials: 8 strided partial sums per column, then 8 adds
+      const int c = tid & (NB - 1), g = tid >> 5;
       T s = T(0);
-      for (int w = 0; w < nwg; ++w) s += part_in[w * NB + tid];
-      s_dots[tid] = s;
+      for (int w0 = g; w0 < nwg; w0 += 64) {
+        T v[8];  // eight independent loads in flight, then a fixed-order sum
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = (w0 + 8 * u < nwg) ? part_in[(w0 + 8 * u) * NB + c] : T(0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+      }
+      s_sum8[g][c] = s;
+      if (tid < NB) s_piv[tid] = (tid < ncol) ? piv_in[tid] : T(0);
     }
     __syncthreads();
-    if (tid == 0) {
-      const T alpha = piv_in[0];
-      const T x2 = s_dots[0];
+    if (tid < NB) {
+      // every one of these lanes derives the reflector scalars from the same sums
+      T x2 = T(0), dot = T(0);
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        x2 += s_sum8[g][0];
+        dot += s_sum8[g][tid];
+      }
+      const T alpha = s_piv[0];
       T beta = alpha, tauv = T(0), scale = T(0);
       if (x2 > T(0)) {
         const T nrm = sqrt(alpha * alpha + x2);
@@ -70,12 +95,13 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
         tauv = (beta - alpha) / beta;
         scale = T(1) / (alpha - beta);
       }
-      s_scal[0] = scale; s_scal[1] = beta; s_scal[2] = tauv;
+      s_tc[tid] = (tid >= 1 && tid < ncol) ? tauv * (s_piv[tid] + scale * dot) : T(0);
+      if (tid == 0) {
+        s_scal[0] = scale; s_scal[1] = beta; s_scal[2] = tauv;
+      }
     }
     __syncthreads();
     const T scale = s_scal[0], beta = s_scal[1], tauv = s_scal[2];
-    if (tid >= 1 && tid < ncol) s_tc[tid] = tauv * (piv_in[tid] + scale * s_dots[tid]);
-    __syncthreads();
     if (live && r >= j) {
       if (r > j) {
         const T v = a[0] * scale;
@@ -127,7 +153,7 @@ __global__ void extract_v_kernel(const T* __restrict__ A, int64_t lda, int nrows
                                  T* __restrict__ Vc, int64_t ldv) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;  // row within the block
   if (i >= nrows) return;
-  for (int c = 0; c < nbw; ++c) {
+  for (int c = blockIdx.y; c < nbw; c += gridDim.y) {
     T v;
     if (i < c) v = T(0);
     else if (i == c) v = T(1);
@@ -136,33 +162,60 @@ __global__ void extract_v_kernel(const T* __restrict__ A, int64_t lda, int nrows
   }
 }
 
-// Compact-WY factor: T upper triangular with H_0 ... H_{nbw-1} = I - V T V^T, from G = V^T V.
-// One wavefront; column i needs the finished columns 0..i-1.
+// Compact-WY factor of up to 32 reflectors: T upper triangular with H_0 ... H_{w-1} = I - V T V^T,
+// from G = V^T V (LAPACK larft, forward / columnwise).  One wavefront per 32-wide diagonal block:
+// blockIdx.x selects the block (G, tau and T advance along the diagonal), so the diagonal blocks
+// of a wider factor are built by one launch.  Column i needs the finished columns 0..i-1; the
+// inner product is unrolled four ways to overlap LDS latency.
 template <typename T>
-__global__ void larft_kernel(const T* __restrict__ G, int ldg, const T* __restrict__ tau, int nbw, T* __restrict__ Tm,
-                             int ldt) {
-  __shared__ T t[64][65];
+__global__ __launch_bounds__(64) void larft32_kernel(const T* __restrict__ G, int ldg, const T* __restrict__ tau,
+                                                      int nbw, T* __restrict__ Tm, int ldt) {
+  __shared__ T t[32][33];
+  __shared__ T g[32][33];
+  const int b = blockIdx.x;
+  const int w = min(32, nbw - 32 * b);
+  G += (int64_t)32 * b * (ldg + 1);
+  Tm += (int64_t)32 * b * (ldt + 1);
+  tau += 32 * b;
   const int k = threadIdx.x;
-  for (int c = 0; c < 64; ++c) t[k][c] = T(0);
-  __syncthreads();
-  for (int i = 0; i < nbw; ++i) {
-    const T ti = tau[i];
-    T s = T(0);
-    if (k < i) {
-      for (int l = k; l < i; ++l) s += t[k][l] * G[l + i * ldg];
-      s = -ti * s;
+  if (k < 32) {
+    for (int c = 0; c < 32; ++c) {
+      t[k][c] = T(0);
+      g[k][c] = (k < w && c < w) ? G[k + c * ldg] : T(0);
     }
+  }
+  __syncthreads();
+  for (int i = 0; i < w; ++i) {
+    const T ti = tau[i];
+    T s0 = T(0), s1 = T(0), s2 = T(0), s3 = T(0);
+    if (k < i) {
+      int l = k;
+      for (; l + 4 <= i; l += 4) {
+        s0 += t[k][l] * g[l][i];
+        s1 += t[k][l + 1] * g[l + 1][i];
+        s2 += t[k][l + 2] * g[l + 2][i];
+        s3 += t[k][l + 3] * g[l + 3][i];
+      }
+      for (; l < i; ++l) s0 += t[k][l] * g[l][i];
+    }
+    const T s = -ti * ((s0 + s1) + (s2 + s3));
     __syncthreads();
     if (k < i) t[k][i] = s;
     if (k == i) t[i][i] = ti;
     __syncthreads();
   }
-  for (int c = 0; c < nbw; ++c)
-    if (k < nbw) Tm[k + c * ldt] = t[k][c];
+  if (k < w)
+    for (int c = 0; c < w; ++c) Tm[k + c * ldt] = t[k][c];
 }
 
-// Finishes the panel columns of the explicit Q: rows above the panel are zero and the unit
-// diagonal of [I; 0] is added to -V (T V1^T).
+template <typename T>
+__global__ void fill_zero_kernel(T* __restrict__ p, int count) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) p[i] = T(0);
+}
+
+// Finishes the block columns [p, p + nbw) of the explicit Q: rows above the block are zero and the
+// unit diagonal of [I; 0] is added to -V (T V1^T).
 template <typename T>
 __global__ void orgqr_panel_fix_kernel(T* __restrict__ Q, int64_t ldq, int p, int nbw) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -173,36 +226,136 @@ __global__ void orgqr_panel_fix_kernel(T* __restrict__ Q, int64_t ldq, int p, in
   }
 }
 
+// ---- block reflectors ------------------------------------------------------------------------
+constexpr int kBrMax = 128;   // widest block reflector (outer block of the QR, back-transformation)
+constexpr int kBrSplits = 8;  // split-K slices of the tall-skinny products
+
+template <typename T>
+struct BlockReflectorWs {
+  T* v;       // n x kBrMax   clean reflector block
+  T* gram;    // kBrMax x kBrMax
+  T* w;       // kBrMax x n
+  T* w2;      // kBrMax x n
+  T* mx;      // kBrMax x kBrMax
+  T* splitk;  // kBrSplits x kBrMax x n
+};
+
+template <typename T, class WS>
+static inline void block_reflector_layout(WS& ws, int64_t n, BlockReflectorWs<T>* out) {
+  BlockReflectorWs<T> b;
+  b.v = ws.template take<T>((size_t)n * kBrMax);
+  b.gram = ws.template take<T>(kBrMax * kBrMax);
+  b.w = ws.template take<T>((size_t)n * kBrMax);
+  b.w2 = ws.template take<T>((size_t)n * kBrMax);
+  b.mx = ws.template take<T>(kBrMax * kBrMax);
+  b.splitk = ws.template take<T>((size_t)kBrSplits * kBrMax * n);
+  if (out) *out = b;
+}
+
+// T (ld kBrMax) from G = V^T V (in ws.gram, ld kBrMax) and tau for nbw <= kBrMax reflectors.  The
+// diagonal 32-blocks [first_block, ...) come from larft32_kernel (earlier ones are already in Tm,
+// the rest of Tm must be zero); block column j then follows from the blocks to its left:
+//   T[0:R, j] = -T[0:R, 0:R] (G[0:R, j] T[j, j]),  R = 32 j.
+template <typename T>
+static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws, int nbw, const T* tau, T* Tm,
+                                    int first_block) {
+  using Skinny = typename SkinnyTile<T>::type;
+  const int blocks = (int)ceil_div64(nbw, 32);
+  if (first_block < blocks) {
+    hipLaunchKernelGGL((larft32_kernel<T>), dim3(blocks - first_block), dim3(64), 0, s,
+                       ws.gram + (int64_t)32 * first_block * (kBrMax + 1), kBrMax, tau + 32 * first_block,
+                       nbw - 32 * first_block, Tm + (int64_t)32 * first_block * (kBrMax + 1), kBrMax);
+    SOAPMI_LAUNCH_CHECK();
+  }
+  for (int j = 1; j < blocks; ++j) {
+    const int R = 32 * j, wj = std::min(32, nbw - R);
+    int rc = gemm<T, Skinny>(s, 0, 0, R, wj, wj, T(1), ws.gram + (int64_t)R * kBrMax, kBrMax,
+                             Tm + (int64_t)R * (kBrMax + 1), kBrMax, T(0), ws.mx, kBrMax);
+    if (rc) return rc;
+    rc = gemm<T, Skinny>(s, 0, 0, R, wj, R, T(-1), Tm, kBrMax, ws.mx, kBrMax, T(0), Tm + (int64_t)R * kBrMax, kBrMax);
+    if (rc) return rc;
+  }
+  return kOk;
+}
+
+template <typename T>
+static inline int gram_of_v(hipStream_t s, const BlockReflectorWs<T>& ws, int rows, int nbw, int64_t ldv) {
+  using Skinny = typename SkinnyTile<T>::type;
+  const int splits = rows >= 2048 ? kBrSplits : 1;
+  if (nbw <= Skinny::BM)
+    return gemm<T, Skinny>(s, 1, 0, nbw, nbw, rows, T(1), ws.v, ldv, ws.v, ldv, T(0), ws.gram, kBrMax, splits,
+                           ws.splitk);
+  return gemm<T>(s, 1, 0, nbw, nbw, rows, T(1), ws.v, ldv, ws.v, ldv, T(0), ws.gram, kBrMax, splits, ws.splitk);
+}
+
+// V (rows x nbw, in ws.v, ld ldv) is in place; computes T (ld kBrMax, fully overwritten) from
+// V^T V and tau.
+template <typename T>
+static inline int build_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws, int rows, int nbw, int64_t ldv,
+                                 const T* tau, T* Tm) {
+  hipLaunchKernelGGL((fill_zero_kernel<T>), dim3(kBrMax * kBrMax / 256), dim3(256), 0, s, Tm, kBrMax * kBrMax);
+  int rc = gram_of_v<T>(s, ws, rows, nbw, ldv);
+  if (rc) return rc;
+  return assemble_t_factor<T>(s, ws, nbw, tau, Tm, 0);
+}
+
+// C (rows x nc, ld ldc) <- C - V op(T) V^T C.
+template <typename T>
+static inline int apply_block_reflector(hipStream_t s, const BlockReflectorWs<T>& ws, const T* Tm, bool transT,
+                                        int rows, int nbw, int nc, int64_t ldv, T* C, int64_t ldc) {
+  using Skinny = typename SkinnyTile<T>::type;
+  using Wide = typename DefaultTile<T>::type;
+  if (nc <= 0 || rows <= 0 || nbw <= 0) return kOk;
+  const bool skinny = nbw <= Skinny::BM;
+  // W = V^T C  (nbw x nc, K = rows): few output tiles, long K -> split-K with a fixed-order reduce
+  const int64_t tiles = ceil_div64(nc, skinny ? Skinny::BN : Wide::BN) * ceil_div64(nbw, skinny ? Skinny::BM : Wide::BM);
+  int splits = 1;
+  if (tiles < 256 && rows >= 1024) splits = (int)std::min<int64_t>(kBrSplits, ceil_div64(512, tiles));
+  int rc;
+  if (skinny) {
+    rc = gemm<T, Skinny>(s, 1, 0, nbw, nc, rows, T(1), ws.v, ldv, C, ldc, T(0), ws.w, kBrMax, splits, ws.splitk);
+    if (rc) return rc;
+    rc = gemm<T, Skinny>(s, transT ? 1 : 0, 0, nbw, nc, nbw, T(1), Tm, kBrMax, ws.w, kBrMax, T(0), ws.w2, kBrMax);
+  } else {
+    rc = gemm<T>(s, 1, 0, nbw, nc, rows, T(1), ws.v, ldv, C, ldc, T(0), ws.w, kBrMax, splits, ws.splitk);
+    if (rc) return rc;
+    rc = gemm<T>(s, transT ? 1 : 0, 0, nbw, nc, nbw, T(1), Tm, kBrMax, ws.w, kBrMax, T(0), ws.w2, kBrMax);
+  }
+  if (rc) return rc;
+  // C -= V W2
+  return gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), ws.v, ldv, ws.w2, kBrMax, T(1), C, ldc);
+}
+
+template <typename T>
+static inline void launch_extract_v(hipStream_t s, const T* A, int64_t lda, int rows, int row0, int col0, int nbw,
+                                    T* V, int64_t ldv) {
+  hipLaunchKernelGGL((extract_v_kernel<T>), dim3((unsigned)ceil_div64(rows, 256), (unsigned)std::min(nbw, 32)),
+                     dim3(256), 0, s, A, lda, rows, row0, col0, nbw, V, ldv);
+}
+
+// ---- QR driver -------------------------------------------------------------------------------
 template <typename T>
 struct QrWorkspace {
-  T* vc;      // n x NB
-  T* t_all;   // panels x NB x NB
+  BlockReflectorWs<T> br;
+  T* t_in;    // kBrMax x kBrMax   factor of the current inner panel
+  T* t_all;   // outer blocks x kBrMax x kBrMax
   T* tau;     // n
-  T* gram;    // NB x NB
-  T* w;       // NB x n
-  T* w2;      // NB x n
-  T* mx;      // NB x NB
   T* part;    // 2 x nwg x NB
   T* piv;     // 2 x NB
-  T* splitk;  // kSplits x NB x n
 };
-constexpr int kQrSplits = 8;
 
 template <typename T, class WS>
 static inline void qr_workspace_layout(WS& ws, int64_t n, QrWorkspace<T>* out) {
-  const int64_t panels = ceil_div64(n, kQrNb);
+  QrWorkspace<T> q;
+  const int64_t blocks = ceil_div64(n, kBrMax);
   const int64_t nwg = ceil_div64(n, 256);
-  T* vc = ws.template take<T>((size_t)n * kQrNb);
-  T* t_all = ws.template take<T>((size_t)panels * kQrNb * kQrNb);
-  T* tau = ws.template take<T>((size_t)n);
-  T* gram = ws.template take<T>(kQrNb * kQrNb);
-  T* w = ws.template take<T>((size_t)n * kQrNb);
-  T* w2 = ws.template take<T>((size_t)n * kQrNb);
-  T* mx = ws.template take<T>(kQrNb * kQrNb);
-  T* part = ws.template take<T>((size_t)2 * nwg * kQrNb);
-  T* piv = ws.template take<T>(2 * kQrNb);
-  T* splitk = ws.template take<T>((size_t)kQrSplits * kQrNb * n);
-  if (out) *out = QrWorkspace<T>{vc, t_all, tau, gram, w, w2, mx, part, piv, splitk};
+  block_reflector_layout<T>(ws, n, out ? &q.br : nullptr);
+  q.t_in = ws.template take<T>(kBrMax * kBrMax);
+  q.t_all = ws.template take<T>((size_t)blocks * kBrMax * kBrMax);
+  q.tau = ws.template take<T>((size_t)n);
+  q.part = ws.template take<T>((size_t)2 * nwg * kQrNb);
+  q.piv = ws.template take<T>(2 * kQrNb);
+  if (out) *out = q;
 }
 
 template <typename T>
@@ -212,77 +365,74 @@ static inline size_t qr_workspace_bytes(int64_t n) {
   return sizer.total();
 }
 
-// Applies the block reflector (or its transpose) of one panel to C (rows x nc, ld ldc) in place:
-// C <- C - Vc op(T) Vc^T C.
-template <typename T>
-static inline int apply_block_reflector(hipStream_t s, const QrWorkspace<T>& ws, const T* Tm, bool transT, int rows,
-                                        int nbw, int nc, int64_t ldv, T* C, int64_t ldc) {
-  using Skinny = typename SkinnyTile<T>::type;
-  if (nc <= 0 || rows <= 0) return kOk;
-  // W = Vc^T C  (nbw x nc, K = rows): few output tiles, long K -> split-K with fixed-order reduce
-  int splits = 1;
-  const int64_t tiles = ceil_div64(nc, Skinny::BN);
-  if (tiles < 256 && rows >= 2048) splits = (int)std::min<int64_t>(kQrSplits, ceil_div64(512, tiles));
-  int rc = gemm<T, Skinny>(s, 1, 0, nbw, nc, rows, T(1), ws.vc, ldv, C, ldc, T(0), ws.w, kQrNb, splits, ws.splitk);
-  if (rc) return rc;
-  // W2 = op(T) W
-  rc = gemm<T, Skinny>(s, transT ? 1 : 0, 0, nbw, nc, nbw, T(1), Tm, kQrNb, ws.w, kQrNb, T(0), ws.w2, kQrNb);
-  if (rc) return rc;
-  // C -= Vc W2
-  return gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), ws.vc, ldv, ws.w2, kQrNb, T(1), C, ldc);
-}
-
 // geqrf in place on A (n x n), then the explicit Q into Qout (n x n).  A is destroyed.
+// Two levels of blocking: 32-column panels (register-resident column steps) are applied only
+// inside their 128-column outer block; the trailing matrix and Q see 128-wide block reflectors,
+// whose products have K = 128 and run on the full-size MFMA tile.
 template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
                                        const QrWorkspace<T>& ws) {
-  using Skinny = typename SkinnyTile<T>::type;
-  const int NB = kQrNb;
-  const int panels = (int)ceil_div64(n, NB);
+  const int NB = kQrNb, OB = kBrMax;
+  const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
+  int rc;
   // ---- factorisation ----
-  for (int pi = 0; pi < panels; ++pi) {
-    const int p = pi * NB, pe = std::min(n, p + NB), nbw = pe - p;
-    const int rows = n - p;
-    const int nwg = (int)ceil_div64(rows, 256);
-    T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
-    T* piv[2] = {ws.piv, ws.piv + NB};
-    for (int j = p - 1; j < pe; ++j) {
-      const int in = (j - p + 1) & 1, out = in ^ 1;
-      hipLaunchKernelGGL((qr_panel_step_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, j, part[in], piv[in],
-                         part[out], piv[out], ws.tau, nwg);
+  for (int bi = 0; bi < blocks; ++bi) {
+    const int P = bi * OB, PE = std::min(n, P + OB), obw = PE - P;
+    T* Tm = ws.t_all + (size_t)bi * OB * OB;
+    hipLaunchKernelGGL((fill_zero_kernel<T>), dim3(OB * OB / 256), dim3(256), 0, s, Tm, OB * OB);
+    int inner_done = 0;
+    for (int p = P; p < PE; p += NB) {
+      const int pe = std::min(PE, p + NB), nbw = pe - p;
+      const int rows = n - p;
+      const int nwg = (int)ceil_div64(rows, 256);
+      T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
+      T* piv[2] = {ws.piv, ws.piv + NB};
+      for (int j = p - 1; j < pe; ++j) {
+        const int in = (j - p + 1) & 1, out = in ^ 1;
+        hipLaunchKernelGGL((qr_panel_step_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, j, part[in],
+                           piv[in], part[out], piv[out], ws.tau, nwg);
+      }
+      SOAPMI_LAUNCH_CHECK();
+      if (pe < PE) {  // the panel's reflectors act on the rest of the outer block only
+        T* Tin = Tm + (int64_t)(p - P) * (OB + 1);  // diagonal block of the outer factor
+        launch_extract_v<T>(s, A, lda, rows, p, p, nbw, ws.br.v, ldv);
+        rc = gram_of_v<T>(s, ws.br, rows, nbw, ldv);
+        if (rc) return rc;
+        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(64), 0, s, ws.br.gram, OB, ws.tau + p, nbw, Tin, OB);
+        SOAPMI_LAUNCH_CHECK();
+        rc = apply_block_reflector<T>(s, ws.br, Tin, true, rows, nbw, PE - pe, ldv, A + p + (int64_t)pe * lda, lda);
+        if (rc) return rc;
+        ++inner_done;
+      }
     }
-    SOAPMI_LAUNCH_CHECK();
-    hipLaunchKernelGGL((extract_v_kernel<T>), dim3((unsigned)ceil_div64(rows, 256)), dim3(256), 0, s, A, lda, rows, p, p, nbw,
-                       ws.vc, ldv);
-    int splits = rows >= 2048 ? kQrSplits : 1;
-    int rc = gemm<T, Skinny>(s, 1, 0, nbw, nbw, rows, T(1), ws.vc, ldv, ws.vc, ldv, T(0), ws.gram, NB, splits, ws.splitk);
+    const int rows = n - P;
+    launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
+    rc = gram_of_v<T>(s, ws.br, rows, obw, ldv);
     if (rc) return rc;
-    T* Tm = ws.t_all + (size_t)pi * NB * NB;
-    hipLaunchKernelGGL((larft_kernel<T>), dim3(1), dim3(64), 0, s, ws.gram, NB, ws.tau + p, nbw, Tm, NB);
-    SOAPMI_LAUNCH_CHECK();
+    rc = assemble_t_factor<T>(s, ws.br, obw, ws.tau + P, Tm, inner_done);
+    if (rc) return rc;
     // trailing columns: C <- H^T C = C - V T^T V^T C
-    rc = apply_block_reflector<T>(s, ws, Tm, true, rows, nbw, n - pe, ldv, A + p + (int64_t)pe * lda, lda);
+    rc = apply_block_reflector<T>(s, ws.br, Tm, true, rows, obw, n - PE, ldv, A + P + (int64_t)PE * lda, lda);
     if (rc) return rc;
   }
-  // ---- explicit Q, panels in reverse ----
-  for (int pi = panels - 1; pi >= 0; --pi) {
-    const int p = pi * NB, pe = std::min(n, p + NB), nbw = pe - p;
-    const int rows = n - p;
-    T* Tm = ws.t_all + (size_t)pi * NB * NB;
-    hipLaunchKernelGGL((extract_v_kernel<T>), dim3((unsigned)ceil_div64(rows, 256)), dim3(256), 0, s, A, lda, rows, p, p, nbw,
-                       ws.vc, ldv);
+  // ---- explicit Q, outer blocks in reverse ----
+  for (int bi = blocks - 1; bi >= 0; --bi) {
+    const int P = bi * OB, PE = std::min(n, P + OB), obw = PE - P;
+    const int rows = n - P;
+    T* Tm = ws.t_all + (size_t)bi * OB * OB;
+    launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
     SOAPMI_LAUNCH_CHECK();
-    // columns to the right already hold Q of the later panels: C <- (I - V T V^T) C
-    int rc = apply_block_reflector<T>(s, ws, Tm, false, rows, nbw, n - pe, ldv, Qout + p + (int64_t)pe * ldq, ldq);
+    // columns to the right already hold Q of the later blocks: C <- (I - V T V^T) C
+    rc = apply_block_reflector<T>(s, ws.br, Tm, false, rows, obw, n - PE, ldv, Qout + P + (int64_t)PE * ldq, ldq);
     if (rc) return rc;
     // own columns: [I;0] - V (T V1^T)
-    rc = gemm<T, Skinny>(s, 0, 1, nbw, nbw, nbw, T(1), Tm, NB, ws.vc, ldv, T(0), ws.mx, NB);
+    rc = gemm<T>(s, 0, 1, obw, obw, obw, T(1), Tm, OB, ws.br.v, ldv, T(0), ws.br.mx, OB);
     if (rc) return rc;
-    rc = gemm<T>(s, 0, 0, rows, nbw, nbw, T(-1), ws.vc, ldv, ws.mx, NB, T(0), Qout + p + (int64_t)p * ldq, ldq);
+    rc = gemm<T>(s, 0, 0, rows, obw, obw, T(-1), ws.br.v, ldv, ws.br.mx, OB, T(0), Qout + P + (int64_t)P * ldq, ldq);
     if (rc) return rc;
-    hipLaunchKernelGGL((orgqr_panel_fix_kernel<T>), dim3((unsigned)ceil_div64(pe, 256)), dim3(256), 0, s, Qout, ldq, p,
-                       nbw);
+    hipLaunchKernelGGL((orgqr_panel_fix_kernel<T>), dim3((unsigned)ceil_div64(PE, 256)), dim3(256), 0, s, Qout, ldq, P,
+                       obw);
     SOAPMI_LAUNCH_CHECK();
   }
   return kOk;

@@ -62,12 +62,13 @@ __device__ __forceinline__ T block_sum_256(T v, T* red) {
   return r;
 }
 
-// alpha2 of the previous column from its partial dots: -1/2 tau (w^T v).
+// Sum of `count` per-workgroup partials, computed by the whole 256-thread workgroup in a fixed
+// order (strided partial sums, then a tree), so every workgroup obtains the same bits.
 template <typename T>
-__device__ __forceinline__ T reduce_partials(const T* part, int count) {
+__device__ __forceinline__ T reduce_partials(const T* __restrict__ part, int count, T* red) {
   T s = T(0);
-  for (int i = 0; i < count; ++i) s += part[i];
-  return s;
+  for (int i = threadIdx.x; i < count; i += 256) s += part[i];
+  return block_sum_256(s, red);
 }
 
 // Kernel A.  Rows r >= j.  i = j - p is the number of reflectors already in the panel.
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(256) void trd_col_update_kernel(T* __restrict__ A, 
   const int r = j + blockIdx.x * 256 + tid;
   const bool live = r < n;
   T alpha2 = T(0);
-  if (i > 0) alpha2 = T(-0.5) * tau[j - 1] * reduce_partials(dot_part, n_dot_part);
+  if (i > 0) alpha2 = T(-0.5) * tau[j - 1] * reduce_partials(dot_part, n_dot_part, red);
   // row j of W and Vc (finalising column i-1 of W on the fly)
   if (tid < i) {
     T wv = W[j + (int64_t)tid * ldw];
@@ -127,11 +128,13 @@ __global__ __launch_bounds__(256) void trd_col_update_kernel(T* __restrict__ A, 
 // Rows of W below the current column that kernel A of this launch did not touch must also be
 // finalised before the rank-2k update; this runs once per panel after its last column.
 template <typename T>
-__global__ void trd_finish_w_kernel(T* __restrict__ W, const T* __restrict__ Vc, int64_t ldw, int n, int row0, int col,
-                                    const T* __restrict__ dot_part, int n_dot_part, const T* __restrict__ tau_prev) {
+__global__ __launch_bounds__(256) void trd_finish_w_kernel(T* __restrict__ W, const T* __restrict__ Vc, int64_t ldw,
+                                                           int n, int row0, int col, const T* __restrict__ dot_part,
+                                                           int n_dot_part, const T* __restrict__ tau_prev) {
+  __shared__ T red[256];
   const int r = row0 + blockIdx.x * blockDim.x + threadIdx.x;
+  const T alpha2 = T(-0.5) * tau_prev[0] * reduce_partials(dot_part, n_dot_part, red);
   if (r >= n) return;
-  const T alpha2 = T(-0.5) * tau_prev[0] * reduce_partials(dot_part, n_dot_part);
   W[r + (int64_t)col * ldw] += alpha2 * Vc[r + (int64_t)col * ldw];
 }
 
@@ -144,11 +147,12 @@ __global__ __launch_bounds__(256) void trd_reflector_kernel(T* __restrict__ A, i
                                                             T* __restrict__ t_part) {
   constexpr int NB = kTrdNb;
   __shared__ T s_red[4][2 * NB];
+  __shared__ T red[256];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int i = j - p;
   const int r = j + 1 + blockIdx.x * 256 + tid;
   const bool live = r < n;
-  const T x2 = reduce_partials(norm_part, n_norm_part);
+  const T x2 = reduce_partials(norm_part, n_norm_part, red);
   const T alpha = A[(j + 1) + (int64_t)j * lda];
   T beta = alpha, tauv = T(0), scale = T(0);
   if (x2 > T(0)) {
@@ -244,15 +248,20 @@ __global__ __launch_bounds__(256) void trd_w_kernel(int n, int p, int j, const T
   constexpr int NB = kTrdNb;
   __shared__ T red[256];
   __shared__ T s_t[2 * NB];
+  __shared__ T s_t4[4][2 * NB];
   const int tid = threadIdx.x;
   const int i = j - p;
   const int r = j + 1 + blockIdx.x * 256 + tid;
-  if (tid < 2 * NB) {
+  {
+    // 2*NB columns x n_t_part partials: 4 strided partial sums per column, then 4 adds
+    const int c = tid & (2 * NB - 1), g0 = tid >> 6;
     T s = T(0);
-    if ((tid % NB) < i)
-      for (int g = 0; g < n_t_part; ++g) s += t_part[(int64_t)g * 2 * NB + tid];
-    s_t[tid] = s;
+    if ((c % NB) < i)
+      for (int g = g0; g < n_t_part; g += 4) s += t_part[(int64_t)g * 2 * NB + c];
+    s_t4[g0][c] = s;
   }
+  __syncthreads();
+  if (tid < 2 * NB) s_t[tid] = (s_t4[0][tid] + s_t4[1][tid]) + (s_t4[2][tid] + s_t4[3][tid]);
   __syncthreads();
   T prod = T(0);
   if (r < n) {
