@@ -194,12 +194,52 @@ __device__ __forceinline__ void store_slab(T* __restrict__ S, const T (&reg)[NV]
   }
 }
 
-template <typename T, class Cfg, class Epi>
+// Fast-path loader state: with full tiles, a K extent that is a multiple of the slab and
+// 16-byte-aligned operands, every thread walks fixed global pointers (one 16-byte load each,
+// bumped by a constant per slab) and fixed LDS offsets; no bounds or layout tests are left in
+// the loop and the operand layout is a template constant.
+template <typename T, int BX, int BK, int NT, int NV, bool XCONTIG>
+struct FastLoader {
+  static constexpr int VW = Vec16<T>::W;
+  using V = typename Vec16<T>::type;
+  const T* ptr[NV];
+  int64_t step;
+  __device__ __forceinline__ void init(const T* base, int64_t ld, int x0, int k0, int tid) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = tid + i * NT;
+      if (XCONTIG) {
+        const int k = v / (BX / VW), xv = v % (BX / VW);
+        ptr[i] = base + (x0 + xv * VW) + (int64_t)(k0 + k) * ld;
+      } else {
+        const int x = v / (BK / VW), kv = v % (BK / VW);
+        ptr[i] = base + (k0 + kv * VW) + (int64_t)(x0 + x) * ld;
+      }
+    }
+    step = XCONTIG ? (int64_t)BK * ld : (int64_t)BK;
+  }
+  __device__ __forceinline__ void load(T (&reg)[NV][VW]) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const V t = *reinterpret_cast<const V*>(ptr[i]);
+      const T* tp = reinterpret_cast<const T*>(&t);
+#pragma unroll
+      for (int e = 0; e < VW; ++e) reg[i][e] = tp[e];
+      ptr[i] += step;
+    }
+  }
+};
+
+// MODE < 0: general path (any size, alignment and layout, tested at run time).
+// MODE in 0..3: fast path, bit 0 = A operand x-contiguous, bit 1 = B operand x-contiguous.
+template <typename T, class Cfg, class Epi, int MODE>
 __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Epi& epi, const int wg, const int z) {
   using MF = Mfma<T>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
   constexpr int MI = Cfg::MI, KI = Cfg::KI, TM = Cfg::TM, TN = Cfg::TN;
   constexpr int SA = Cfg::SA, SB = Cfg::SB, VW = Cfg::VW;
+  constexpr bool FAST = MODE >= 0;
+  constexpr bool AXC = (MODE & 1) != 0, BXC = (MODE & 2) != 0;
 
   __shared__ __attribute__((aligned(16))) T As[2][BK * SA];
   __shared__ __attribute__((aligned(16))) T Bs[2][BK * SB];
@@ -242,12 +282,22 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
       for (int r = 0; r < MF::NACC; ++r) acc[i][j][r] = T(0);
 
   T ra[Cfg::NVA][VW], rb[Cfg::NVB][VW];
-  const bool a_xc = !p.transA, b_xc = (p.transB != 0);
+  const bool a_xc = FAST ? AXC : !p.transA;
+  const bool b_xc = FAST ? BXC : (p.transB != 0);
   const int nk = (kend - kbeg + BK - 1) / BK;
+  FastLoader<T, BM, BK, NT, Cfg::NVA, AXC> fa;
+  FastLoader<T, BN, BK, NT, Cfg::NVB, BXC> fb;
 
   if (nk > 0) {
-    load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, kbeg, kend, a_xc, p.vecA, tid);
-    load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, kbeg, kend, b_xc, p.vecB, tid);
+    if (FAST) {
+      fa.init(p.A, p.lda, m0, kbeg, tid);
+      fb.init(p.B, p.ldb, n0, kbeg, tid);
+      fa.load(ra);
+      fb.load(rb);
+    } else {
+      load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, kbeg, kend, a_xc, p.vecA, tid);
+      load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, kbeg, kend, b_xc, p.vecB, tid);
+    }
     store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[0], ra, a_xc, tid);
     store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[0], rb, b_xc, tid);
   }
@@ -257,9 +307,14 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < nk) {
-      const int k0 = kbeg + (kt + 1) * BK;
-      load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, k0, kend, a_xc, p.vecA, tid);
-      load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, k0, kend, b_xc, p.vecB, tid);
+      if (FAST) {
+        fa.load(ra);
+        fb.load(rb);
+      } else {
+        const int k0 = kbeg + (kt + 1) * BK;
+        load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, k0, kend, a_xc, p.vecA, tid);
+        load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, k0, kend, b_xc, p.vecB, tid);
+      }
     }
     const T* as = As[buf];
     const T* bs = Bs[buf];
@@ -291,15 +346,15 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
 #pragma unroll
       for (int r = 0; r < MF::NACC; ++r) {
         const int n = n0 + wn0 + j * MI + MF::acc_row(r, lane);
-        if (m < p.M && n < p.N) epi(m, n, acc[i][j][r], z);
+        if (FAST || (m < p.M && n < p.N)) epi(m, n, acc[i][j][r], z);
       }
     }
   }
 }
 
-template <typename T, class Cfg, class Epi>
+template <typename T, class Cfg, class Epi, int MODE>
 __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi) {
-  gemm_tile_body<T, Cfg, Epi>(p, epi, blockIdx.x, blockIdx.y);
+  gemm_tile_body<T, Cfg, Epi, MODE>(p, epi, blockIdx.x, blockIdx.y);
 }
 
 // One problem per blockIdx.z, described in device memory (sizes may be produced by earlier
@@ -313,7 +368,7 @@ template <typename T, class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void gemm_batched_kernel(const BatchedGemm<T>* __restrict__ batch) {
   const BatchedGemm<T> b = batch[blockIdx.z];
   if (b.p.M <= 0 || b.p.N <= 0) return;
-  gemm_tile_body<T, Cfg, EpiStore<T>>(b.p, b.e, blockIdx.x, 0);
+  gemm_tile_body<T, Cfg, EpiStore<T>, -1>(b.p, b.e, blockIdx.x, 0);
 }
 
 // Device-side twin of make_problem for the default tile.
@@ -403,7 +458,16 @@ static inline int launch_gemm(hipStream_t stream, const GemmProblem<T>& p, const
   if (p.M <= 0 || p.N <= 0) return kOk;
   const int chunk = (p.num_tiles + 7) / 8;
   dim3 grid(8 * chunk, k_splits, 1);
-  hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi>), grid, dim3(Cfg::NT), 0, stream, p, epi);
+  const bool fast = p.vecA && p.vecB && p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K > 0 &&
+                    p.K % Cfg::BK == 0 && p.k_chunk % Cfg::BK == 0 && p.K % p.k_chunk == 0;
+  const int mode = fast ? ((p.transA ? 0 : 1) | (p.transB ? 2 : 0)) : -1;
+  switch (mode) {
+    case 0: hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi, 0>), grid, dim3(Cfg::NT), 0, stream, p, epi); break;
+    case 1: hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi, 1>), grid, dim3(Cfg::NT), 0, stream, p, epi); break;
+    case 2: hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi, 2>), grid, dim3(Cfg::NT), 0, stream, p, epi); break;
+    case 3: hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi, 3>), grid, dim3(Cfg::NT), 0, stream, p, epi); break;
+    default: hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi, -1>), grid, dim3(Cfg::NT), 0, stream, p, epi); break;
+  }
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
