@@ -146,6 +146,148 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
   if (tid < NB) part_out[blockIdx.x * NB + tid] = s_wave[0][tid] + s_wave[1][tid] + s_wave[2][tid] + s_wave[3][tid];
 }
 
+// ---- whole panel in one launch -----------------------------------------------------------------
+// The same column recurrence as qr_panel_step_kernel, but the 32 columns of a panel run inside
+// one launch: every thread keeps its row of the panel in registers from the first column to the
+// last (loaded once, each finished column stored once), and the workgroups meet at a counter in
+// device memory between columns.  Requirements: all workgroups of the launch are resident at the
+// same time (the host launches at most kQrPersistentMaxWg of them, one per CU), and the counter
+// starts the launch at `base`.  Waiting is bounded: a workgroup that does not see the others
+// arrive within kQrSpinLimit polls raises `error` and leaves, and so does everyone who sees the flag.
+constexpr int kQrPersistentMaxWg = 128;
+constexpr unsigned kQrSpinLimit = 1u << 22;
+
+__device__ __forceinline__ bool panel_grid_barrier(unsigned* counter, unsigned target, int* error, int* s_fail) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // The release covers this wavefront's own earlier stores, which is why every global value the
+    // other workgroups read after the barrier is written by wavefront 0.
+    __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    int fail = 0;
+    unsigned spins = 0;
+    while (__hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      if (++spins > kQrSpinLimit || __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+        fail = 1;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+    if (fail) __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *s_fail = fail;
+  }
+  __syncthreads();
+  return *s_fail == 0;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void qr_panel_persistent_kernel(T* __restrict__ A, int64_t lda, int n, int p, int pe,
+                                                                  T* part, T* piv, T* __restrict__ tau,
+                                                                  unsigned* counter, unsigned base, int* error,
+                                                                  int nwg) {
+  constexpr int NB = kQrNb;
+  __shared__ T s_tc[NB];
+  __shared__ T s_wave[4][NB];
+  __shared__ T s_sum8[8][NB];
+  __shared__ T s_piv[NB];
+  __shared__ T s_scal[3];
+  __shared__ int s_fail;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wg = blockIdx.x;
+  const int r = p + wg * 256 + tid;
+  const int nbw = pe - p;
+  const bool live = r < n;
+
+  T a[NB];  // a[k] = A[r, j + k] for the current column j: the row is shifted left after each column
+#pragma unroll
+  for (int c = 0; c < NB; ++c) a[c] = (live && c < nbw) ? A[r + (int64_t)(p + c) * lda] : T(0);
+
+  for (int c = 0; c < nbw; ++c) {
+    const int j = p + c;
+    T* part_c = part + (size_t)(c & 1) * nwg * NB;
+    T* piv_c = piv + (c & 1) * NB;
+    // dot products of column j with the remaining panel columns over the rows below the pivot
+    {
+      const bool below = live && r > j;
+      T vals[NB];
+#pragma unroll
+      for (int k = 0; k < NB; ++k) vals[k] = below ? a[0] * a[k] : T(0);
+      const T total = wave_reduce_32<T>(vals, lane);
+      if ((lane & 1) == 0) s_wave[wave][(lane >> 1) & 31] = total;
+      if (live && r == j) {
+#pragma unroll
+        for (int k = 0; k < NB; ++k) s_piv[k] = a[k];
+      }
+    }
+    __syncthreads();
+    if (tid < NB) {
+      const T sum = (s_wave[0][tid] + s_wave[1][tid]) + (s_wave[2][tid] + s_wave[3][tid]);
+      __hip_atomic_store(part_c + wg * NB + tid, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (j >= p + wg * 256 && j < p + wg * 256 + 256)  // this workgroup owns the pivot row
+        __hip_atomic_store(piv_c + tid, s_piv[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (!panel_grid_barrier(counter, base + (unsigned)nwg * (unsigned)(c + 1), error, &s_fail)) return;
+    {
+      // fixed-order sum of the per-workgroup partials, as in qr_panel_step_kernel
+      const int k = tid & (NB - 1), g = tid >> 5;
+      T s = T(0);
+      for (int w0 = g; w0 < nwg; w0 += 64) {
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          v[u] = (w0 + 8 * u < nwg)
+                     ? __hip_atomic_load(part_c + (w0 + 8 * u) * NB + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                     : T(0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+      }
+      s_sum8[g][k] = s;
+      if (tid < NB) s_piv[tid] = __hip_atomic_load(piv_c + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (tid < NB) {
+      T x2 = T(0), dot = T(0);
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        x2 += s_sum8[g][0];
+        dot += s_sum8[g][tid];
+      }
+      const T alpha = s_piv[0];
+      T beta = alpha, tauv = T(0), scale = T(0);
+      if (x2 > T(0)) {
+        const T nrm = sqrt(alpha * alpha + x2);
+        beta = (alpha >= T(0)) ? -nrm : nrm;
+        tauv = (beta - alpha) / beta;
+        scale = T(1) / (alpha - beta);
+      }
+      s_tc[tid] = (tid >= 1) ? tauv * (s_piv[tid] + scale * dot) : T(0);
+      if (tid == 0) {
+        s_scal[0] = scale; s_scal[1] = beta; s_scal[2] = tauv;
+      }
+    }
+    __syncthreads();
+    const T scale = s_scal[0], beta = s_scal[1], tauv = s_scal[2];
+    if (live && r >= j) {
+      if (r > j) {
+        const T v = a[0] * scale;
+        a[0] = v;
+#pragma unroll
+        for (int k = 1; k < NB; ++k) a[k] -= s_tc[k] * v;
+      } else {
+        a[0] = beta;
+#pragma unroll
+        for (int k = 1; k < NB; ++k) a[k] -= s_tc[k];
+        tau[j] = tauv;
+      }
+    }
+    if (live) A[r + (int64_t)j * lda] = a[0];  // column j is final
+#pragma unroll
+    for (int k = 0; k + 1 < NB; ++k) a[k] = a[k + 1];
+    a[NB - 1] = T(0);
+    // s_piv, s_wave are rewritten only after the next __syncthreads pair; s_tc is read above
+    __syncthreads();
+  }
+}
+
 // Vc (nrows x nbw, ld ldv) <- the unit-lower-trapezoidal reflector block stored in A with its
 // unit diagonal at (row0 + c, col0 + c): zeros above, ones on, A below.
 template <typename T>
@@ -206,6 +348,13 @@ __global__ __launch_bounds__(64) void larft32_kernel(const T* __restrict__ G, in
   }
   if (k < w)
     for (int c = 0; c < w; ++c) Tm[k + c * ldt] = t[k][c];
+}
+
+// Fills the diagonal of Q with NaN if the error flag is set.
+template <typename T>
+__global__ void poison_on_error_kernel(T* __restrict__ Q, int64_t ldq, int n, const int* __restrict__ error) {
+  if (*error == 0) return;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) Q[i + (int64_t)i * ldq] = T(NAN);
 }
 
 template <typename T>
@@ -342,6 +491,7 @@ struct QrWorkspace {
   T* tau;     // n
   T* part;    // 2 x nwg x NB
   T* piv;     // 2 x NB
+  unsigned* sync;  // [0] arrival counter of the persistent panel kernel, [1] its error flag
 };
 
 template <typename T, class WS>
@@ -355,6 +505,7 @@ static inline void qr_workspace_layout(WS& ws, int64_t n, QrWorkspace<T>* out) {
   q.tau = ws.template take<T>((size_t)n);
   q.part = ws.template take<T>((size_t)2 * nwg * kQrNb);
   q.piv = ws.template take<T>(2 * kQrNb);
+  q.sync = ws.template take<unsigned>(64);
   if (out) *out = q;
 }
 
@@ -376,6 +527,8 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
   int rc;
+  unsigned sync_base = 0;
+  hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
   // ---- factorisation ----
   for (int bi = 0; bi < blocks; ++bi) {
     const int P = bi * OB, PE = std::min(n, P + OB), obw = PE - P;
@@ -388,10 +541,16 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       const int nwg = (int)ceil_div64(rows, 256);
       T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
       T* piv[2] = {ws.piv, ws.piv + NB};
-      for (int j = p - 1; j < pe; ++j) {
-        const int in = (j - p + 1) & 1, out = in ^ 1;
-        hipLaunchKernelGGL((qr_panel_step_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, j, part[in],
-                           piv[in], part[out], piv[out], ws.tau, nwg);
+      if (nwg <= kQrPersistentMaxWg) {
+        hipLaunchKernelGGL((qr_panel_persistent_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.part,
+                           ws.piv, ws.tau, ws.sync, sync_base, reinterpret_cast<int*>(ws.sync + 1), nwg);
+        sync_base += (unsigned)nwg * (unsigned)nbw;
+      } else {
+        for (int j = p - 1; j < pe; ++j) {
+          const int in = (j - p + 1) & 1, out = in ^ 1;
+          hipLaunchKernelGGL((qr_panel_step_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, j, part[in],
+                             piv[in], part[out], piv[out], ws.tau, nwg);
+        }
       }
       SOAPMI_LAUNCH_CHECK();
       if (pe < PE) {  // the panel's reflectors act on the rest of the outer block only
@@ -435,6 +594,10 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
                        obw);
     SOAPMI_LAUNCH_CHECK();
   }
+  // A panel kernel that gave up waiting leaves garbage behind: make that impossible to miss.
+  hipLaunchKernelGGL((poison_on_error_kernel<T>), dim3(1), dim3(64), 0, s, Qout, ldq, n,
+                     reinterpret_cast<const int*>(ws.sync + 1));
+  SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
 
