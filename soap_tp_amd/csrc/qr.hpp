@@ -427,10 +427,21 @@ static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws
   return kOk;
 }
 
+// Number of K slices for a tall-skinny product with `tiles` output tiles, K = rows, an M x N
+// output: enough slices to occupy the chip (about 512 workgroups), at least 256 rows each, and no
+// more partial results than the split-K buffer (kBrSplits * kBrMax * ldv elements) holds.
+static inline int split_count(int64_t tiles, int rows, int M, int N, int64_t ldv) {
+  if (rows < 1024) return 1;
+  int64_t splits = std::min<int64_t>(ceil_div64(512, tiles), rows / 256);
+  const int64_t capacity = (int64_t)kBrSplits * kBrMax * ldv / std::max<int64_t>(1, (int64_t)M * N);
+  splits = std::min<int64_t>(splits, std::min<int64_t>(capacity, 64));
+  return (int)std::max<int64_t>(splits, 1);
+}
+
 template <typename T>
 static inline int gram_of_v(hipStream_t s, const BlockReflectorWs<T>& ws, int rows, int nbw, int64_t ldv) {
   using Skinny = typename SkinnyTile<T>::type;
-  const int splits = rows >= 2048 ? kBrSplits : 1;
+  const int splits = split_count(1, rows, nbw, nbw, ldv);
   if (nbw <= Skinny::BM)
     return gemm<T, Skinny>(s, 1, 0, nbw, nbw, rows, T(1), ws.v, ldv, ws.v, ldv, T(0), ws.gram, kBrMax, splits,
                            ws.splitk);
@@ -458,8 +469,7 @@ static inline int apply_block_reflector(hipStream_t s, const BlockReflectorWs<T>
   const bool skinny = nbw <= Skinny::BM;
   // W = V^T C  (nbw x nc, K = rows): few output tiles, long K -> split-K with a fixed-order reduce
   const int64_t tiles = ceil_div64(nc, skinny ? Skinny::BN : Wide::BN) * ceil_div64(nbw, skinny ? Skinny::BM : Wide::BM);
-  int splits = 1;
-  if (tiles < 256 && rows >= 1024) splits = (int)std::min<int64_t>(kBrSplits, ceil_div64(512, tiles));
+  const int splits = split_count(tiles, rows, nbw, nc, ldv);
   int rc;
   if (skinny) {
     rc = gemm<T, Skinny>(s, 1, 0, nbw, nc, rows, T(1), ws.v, ldv, C, ldc, T(0), ws.w, kBrMax, splits, ws.splitk);
