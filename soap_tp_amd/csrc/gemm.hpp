@@ -410,11 +410,11 @@ template <typename T>
 struct DefaultTile;
 template <>
 struct DefaultTile<float> {
-  using type = GemmTile<float, 128, 128, 16, 2, 2>;
+  using type = GemmTile<float, 128, 128, 16, 4, 2>;
 };
 template <>
 struct DefaultTile<double> {
-  using type = GemmTile<double, 128, 128, 8, 2, 2>;
+  using type = GemmTile<double, 128, 128, 16, 4, 2>;
 };
 
 // Tile for products whose M extent is a panel width (32): tall-skinny block-reflector work.
