@@ -32,9 +32,11 @@ HBM_PEAK_GBS = 8000.0
 GRID = (1, 1)
 HYPER = dict(preconditioner_beta=0.95, beta1=0.95, beta2=0.95, eps=1e-8, basis_refresh_interval=10)
 
-# HBM bytes per launch of the rotation product, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script (see profiles/); keyed by shape.  None until measured for a shape.
-MEASURED_TRAFFIC_BYTES = {}
+# Memory bytes per launch of the rotation product (mean of the four launches of a step), from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of tests/native/abi_probe.bin, each scaled by what the
+# same counter reads for a layout copy of known size; summary under profiles/.  Keyed by shape; a shape
+# that has not been measured reports null.
+MEASURED_TRAFFIC_BYTES = {"4096x11008": 5.33e9}
 
 
 def device_low_rank_plus_noise(rows, columns, rank, seed, device, noise_std=1e-4):
@@ -168,6 +170,16 @@ def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True):
     }
 
 
+def calibration_copies(rows, columns, count, device):
+    """Row-major to column-major copies of a rows x columns fp32 matrix through the library."""
+    from soap_tp_amd.ops import redistribute_tp_shard_to_2d_block_cyclic
+
+    source = torch.randn(rows, columns, device=device)
+    for _ in range(count):
+        redistribute_tp_shard_to_2d_block_cyclic(source, (rows, columns), 128, GRID, shard_dim=1)
+    torch.cuda.synchronize()
+
+
 def parse_shape(text):
     rows, columns = text.lower().split("x")
     return int(rows), int(columns)
@@ -182,6 +194,10 @@ def main():
     parser.add_argument("--rank", type=int, default=128)
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-other-shapes", action="store_true")
+    parser.add_argument("--calibration-copies", type=int, default=0,
+                        help="run this many layout copies of one rows x columns fp32 matrix (transpose_kernel: "
+                             "4*rows*columns bytes read and as many written) before the schedule; the known-size "
+                             "kernel that hardware-counter readings of a profiled run are scaled by")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the SOAP step: this build has no multi-GPU path, "
@@ -194,6 +210,8 @@ def main():
     torch.cuda.set_device(device)
     rows, columns = args.shape
 
+    if args.calibration_copies > 0:
+        calibration_copies(rows, columns, args.calibration_copies, device)
     main_run = run_schedule(args.shape, args.rank, args.steps, args.warmup, device)
     ms_per_step = main_run["total_ms"] / args.steps
     rotation_flops = 4.0 * rows * columns * (rows + columns)
@@ -237,6 +255,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
             "traffic": traffic,
+            "traffic_unit": "bytes per launch (L2 fills + writes; compulsory 0.82e9)",
             "flops_per_step": rotation_flops,
             "avg_launch_ms": main_run["rotate_ms"] / 4.0,
             "gram_pair_tflops_syrk_convention": gram_flops / (main_run["gram_ms"] * 1e-3) / 1e12,

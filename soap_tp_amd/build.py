@@ -14,6 +14,11 @@ from pathlib import Path
 PACKAGE_DIR = Path(__file__).resolve().parent
 CSRC_DIR = PACKAGE_DIR / "csrc"
 LIBRARY_PATH = PACKAGE_DIR / "libsoap_mi355.so"
+INCLUDE_DIR = PACKAGE_DIR.parent / "include"
+# A C++ program that calls the C ABI without Python or torch (used by a GPU test and for
+# hardware-counter runs, where the profiled program should be a plain executable).
+ABI_PROBE_SOURCE = PACKAGE_DIR.parent / "tests" / "native" / "abi_probe.cpp"
+ABI_PROBE_PATH = PACKAGE_DIR.parent / "tests" / "native" / "abi_probe.bin"
 SOURCES = ("api.hip",)
 
 # -packed-fp32-ops is switched off on purpose: the compiler must not fuse scalar fp32 code
@@ -52,5 +57,19 @@ def build(verbose: bool = False) -> Path:
     return LIBRARY_PATH
 
 
+def build_abi_probe(verbose: bool = False) -> Path:
+    """Host-only build of tests/native/abi_probe.cpp against the shared library."""
+    command = [hipcc_path(), "-O2", "-std=c++17", "-I", str(INCLUDE_DIR), str(ABI_PROBE_SOURCE),
+               "-L", str(PACKAGE_DIR), "-lsoap_mi355", "-Wl,-rpath,$ORIGIN/../../soap_tp_amd",
+               "-Wno-unused-result", "-o", str(ABI_PROBE_PATH)]
+    if verbose:
+        print(" ".join(command), flush=True)
+    completed = subprocess.run(command, capture_output=True, text=True)
+    if completed.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({completed.returncode}):\n{completed.stderr}")
+    return ABI_PROBE_PATH
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_abi_probe(verbose=True))

@@ -16,6 +16,10 @@
 #pragma once
 #include "common.hpp"
 
+#ifndef SOAPMI_TILE_GROUP_ROWS
+#define SOAPMI_TILE_GROUP_ROWS 8
+#endif
+
 namespace soapmi {
 
 template <typename T>
@@ -258,10 +262,11 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
     tm = bi;
     tn = t - bi * (bi + 1) / 2;
   } else {
-    const int per = 8 * p.tiles_n;
+    constexpr int GR = SOAPMI_TILE_GROUP_ROWS;
+    const int per = GR * p.tiles_n;
     const int g = t / per, r = t - g * per;
-    const int rows = min(8, p.tiles_m - g * 8);
-    tm = g * 8 + r % rows;
+    const int rows = min(GR, p.tiles_m - g * GR);
+    tm = g * GR + r % rows;
     tn = r / rows;
   }
   const int m0 = tm * BM, n0 = tn * BN;

@@ -17,6 +17,7 @@
 #pragma once
 #include "common.hpp"
 #include "gemm.hpp"
+#include "qr.hpp"
 
 namespace soapmi {
 
@@ -101,17 +102,26 @@ __global__ __launch_bounds__(256) void trd_col_update_kernel(T* __restrict__ A, 
   __syncthreads();
   T x2 = T(0);
   if (live) {
+    // all 2*NB loads are issued before the first use (fixed trip count, guarded by k < i)
+    T wr[NB], vr[NB];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
+      vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
+    }
     T acc = T(0);
-    for (int k = 0; k < i; ++k) {
-      T wr = W[r + (int64_t)k * ldw];
-      const T vr = Vc[r + (int64_t)k * ldw];
-      if (k == i - 1) {
-        wr += alpha2 * vr;
-        // Row j stays unfinished in memory: every workgroup reads it above and adds alpha2
-        // itself, and no later column looks at row j of W again.
-        if (r != j) W[r + (int64_t)k * ldw] = wr;
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      if (k < i) {
+        T wk = wr[k];
+        if (k == i - 1) {
+          wk += alpha2 * vr[k];
+          // Row j stays unfinished in memory: every workgroup reads it above and adds alpha2
+          // itself, and no later column looks at row j of W again.
+          if (r != j) W[r + (int64_t)k * ldw] = wk;
+        }
+        acc += vr[k] * s_wj[k] + wk * s_vj[k];
       }
-      acc += vr * s_wj[k] + wr * s_vj[k];
     }
     T a = A[r + (int64_t)j * lda];
     if (i > 0) {
@@ -184,16 +194,22 @@ __global__ __launch_bounds__(256) void trd_reflector_kernel(T* __restrict__ A, i
   if (blockIdx.x == 0) {
     for (int rr = p + tid; rr <= j; rr += 256) Vc[rr + (int64_t)i * ldw] = T(0);
   }
-  // partial W^T v and V^T v over this workgroup's rows (columns k < i)
-  for (int k0 = 0; k0 < 2 * i; k0 += 1) {
-    const int k = k0 >> 1;
-    const bool useW = (k0 & 1) == 0;
-    T prod = T(0);
-    if (live) prod = (useW ? W[r + (int64_t)k * ldw] : Vc[r + (int64_t)k * ldw]) * v;
-    // wavefront reduction
+  // partial W^T v and V^T v over this workgroup's rows (columns k < i): 2*NB products per thread,
+  // two 32-value butterflies per wavefront
+  {
+    T pw[NB], pv[NB];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) prod += __shfl_xor(prod, off, 64);
-    if (lane == 0) s_red[wave][(useW ? 0 : NB) + k] = prod;
+    for (int k = 0; k < NB; ++k) {
+      const bool on = live && k < i;
+      pw[k] = on ? W[r + (int64_t)k * ldw] * v : T(0);
+      pv[k] = on ? Vc[r + (int64_t)k * ldw] * v : T(0);
+    }
+    const T tw = wave_reduce_32<T>(pw, lane);
+    const T tv = wave_reduce_32<T>(pv, lane);
+    if ((lane & 1) == 0) {
+      s_red[wave][(lane >> 1) & 31] = tw;
+      s_red[wave][NB + ((lane >> 1) & 31)] = tv;
+    }
   }
   __syncthreads();
   if (tid < 2 * NB) {
@@ -265,10 +281,20 @@ __global__ __launch_bounds__(256) void trd_w_kernel(int n, int p, int j, const T
   __syncthreads();
   T prod = T(0);
   if (r < n) {
+    T yp[kTrdMaxChunks], wr[NB], vr[NB];
+#pragma unroll
+    for (int c = 0; c < kTrdMaxChunks; ++c) yp[c] = (c < n_chunks) ? y_part[(int64_t)c * n + r] : T(0);
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
+      wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
+    }
     T y = T(0);
-    for (int c = 0; c < n_chunks; ++c) y += y_part[(int64_t)c * n + r];
+#pragma unroll
+    for (int c = 0; c < kTrdMaxChunks; ++c) y += yp[c];
     T corr = T(0);
-    for (int k = 0; k < i; ++k) corr += Vc[r + (int64_t)k * ldw] * s_t[k] + W[r + (int64_t)k * ldw] * s_t[NB + k];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) corr += vr[k] * s_t[k] + wr[k] * s_t[NB + k];
     const T wv = tau[j] * (y - corr);
     W[r + (int64_t)i * ldw] = wv;
     prod = wv * Vc[r + (int64_t)i * ldw];

@@ -1,0 +1,135 @@
+// Stand-alone caller of the C ABI: no Python, no torch, only the HIP runtime for device memory.
+//
+//   abi_probe [rows cols [repeats [copies]]]
+//
+// 1. `copies` layout copies of a rows x cols fp32 matrix (4*rows*cols bytes read, as many written):
+//    the kernel of known size that hardware-counter readings of a profiled run are scaled by.
+// 2. `repeats` calls of soapmi_rotate_adam_rotate_f32 (the update half of a steady-state step, four
+//    MFMA products) with identity bases, so that the expected result is plain Adam on the gradient
+//    and a sample of entries can be checked on the host in closed form.
+// Prints the average time per call and the rate over the 4*rows*cols*(rows+cols) algorithmic flops;
+// exits non-zero if any call fails or the sampled entries are off.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "soap_mi355.h"
+
+#define HIP_OK(expr)                                                                      \
+  do {                                                                                    \
+    hipError_t status_ = (expr);                                                          \
+    if (status_ != hipSuccess) {                                                          \
+      std::fprintf(stderr, "%s failed: %s\n", #expr, hipGetErrorString(status_));        \
+      return 2;                                                                           \
+    }                                                                                     \
+  } while (0)
+
+#define ABI_OK(expr)                                                                      \
+  do {                                                                                    \
+    int status_ = (expr);                                                                 \
+    if (status_ != SOAPMI_OK) {                                                           \
+      std::fprintf(stderr, "%s returned %d: %s\n", #expr, status_, soapmi_last_error()); \
+      return 3;                                                                           \
+    }                                                                                     \
+  } while (0)
+
+static float host_value(uint64_t index) {
+  // cheap reproducible pseudo-random value in (-0.5, 0.5)
+  uint64_t x = index * 0x9E3779B97F4A7C15ull + 0x632BE59BD9B4E019ull;
+  x ^= x >> 29;
+  x *= 0xBF58476D1CE4E5B9ull;
+  x ^= x >> 32;
+  return (float)((double)(x & 0xFFFFFF) / (double)0x1000000 - 0.5);
+}
+
+int main(int argc, char** argv) {
+  const int64_t rows = argc > 2 ? std::atoll(argv[1]) : 4096;
+  const int64_t cols = argc > 2 ? std::atoll(argv[2]) : 11008;
+  const int repeats = argc > 3 ? std::atoi(argv[3]) : 5;
+  const int copies = argc > 4 ? std::atoi(argv[4]) : 3;
+  if (rows <= 0 || cols <= 0 || repeats <= 0 || copies < 0) {
+    std::fprintf(stderr, "usage: abi_probe [rows cols [repeats [copies]]]\n");
+    return 1;
+  }
+  std::printf("backend %s, %lld x %lld, %d calls, %d calibration copies\n", soapmi_compiled_gpu_backend(),
+              (long long)rows, (long long)cols, repeats, copies);
+  std::fflush(stdout);
+
+  const size_t mn = (size_t)rows * cols;
+  std::vector<float> gradient(mn);
+  for (size_t i = 0; i < mn; ++i) gradient[i] = host_value(i);
+  std::vector<float> identity_l((size_t)rows * rows, 0.0f), identity_r((size_t)cols * cols, 0.0f);
+  for (int64_t i = 0; i < rows; ++i) identity_l[(size_t)i * rows + i] = 1.0f;
+  for (int64_t i = 0; i < cols; ++i) identity_r[(size_t)i * cols + i] = 1.0f;
+
+  float *d_gradient, *d_update, *d_ql, *d_qr, *d_momentum, *d_variance, *d_copy;
+  void* d_workspace;
+  const size_t workspace_bytes = soapmi_rotate_adam_rotate_workspace_bytes(rows, cols);
+  HIP_OK(hipMalloc((void**)&d_gradient, mn * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_update, mn * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_copy, mn * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_momentum, mn * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_variance, mn * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_ql, identity_l.size() * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_qr, identity_r.size() * sizeof(float)));
+  HIP_OK(hipMalloc(&d_workspace, workspace_bytes));
+  HIP_OK(hipMemcpy(d_gradient, gradient.data(), mn * sizeof(float), hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_ql, identity_l.data(), identity_l.size() * sizeof(float), hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_qr, identity_r.data(), identity_r.size() * sizeof(float), hipMemcpyHostToDevice));
+  HIP_OK(hipMemset(d_momentum, 0, mn * sizeof(float)));
+  HIP_OK(hipMemset(d_variance, 0, mn * sizeof(float)));
+
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  for (int c = 0; c < copies; ++c)
+    ABI_OK(soapmi_row_major_to_col_major_f32(d_gradient, cols, d_copy, rows, rows, cols, stream));
+
+  const double beta1 = 0.95, beta2 = 0.95, eps = 1e-8;
+  hipEvent_t begin, end;
+  HIP_OK(hipEventCreate(&begin));
+  HIP_OK(hipEventCreate(&end));
+  // first call untimed (step 1), then `repeats` timed calls (steps 2 ..)
+  ABI_OK(soapmi_rotate_adam_rotate_f32(d_gradient, cols, d_update, cols, d_ql, rows, d_qr, cols, d_momentum, rows,
+                                       d_variance, rows, rows, cols, 1, beta1, beta2, eps, d_workspace,
+                                       workspace_bytes, stream));
+  HIP_OK(hipEventRecord(begin, stream));
+  for (int r = 0; r < repeats; ++r)
+    ABI_OK(soapmi_rotate_adam_rotate_f32(d_gradient, cols, d_update, cols, d_ql, rows, d_qr, cols, d_momentum, rows,
+                                         d_variance, rows, rows, cols, 2 + r, beta1, beta2, eps, d_workspace,
+                                         workspace_bytes, stream));
+  HIP_OK(hipEventRecord(end, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  float elapsed_ms = 0.0f;
+  HIP_OK(hipEventElapsedTime(&elapsed_ms, begin, end));
+  const double per_call_ms = elapsed_ms / repeats;
+  const double flops = 4.0 * (double)rows * (double)cols * (double)(rows + cols);
+  std::printf("rotate_adam_rotate: %.3f ms per call, %.1f TFLOP/s over 4mn(m+n) flops\n", per_call_ms,
+              flops / (per_call_ms * 1e-3) / 1e12);
+
+  // With identity bases and a constant gradient g, after t steps m = (1-b1^t) g, v = (1-b2^t) g^2,
+  // so the update is g / (|g| + eps / sqrt(1-b2^t)) for every entry.
+  std::vector<float> update(mn);
+  HIP_OK(hipMemcpy(update.data(), d_update, mn * sizeof(float), hipMemcpyDeviceToHost));
+  const int steps = 1 + repeats;
+  const double bc2 = 1.0 - std::pow(beta2, steps);
+  double worst = 0.0;
+  const size_t stride = mn / 4099 + 1;
+  for (size_t i = 0; i < mn; i += stride) {
+    const double g = gradient[i];
+    const double expected = g / (std::fabs(g) + eps / std::sqrt(bc2));
+    worst = std::fmax(worst, std::fabs((double)update[i] - expected));
+  }
+  std::printf("closed-form check on %zu sampled entries: max abs error %.3e\n", (mn + stride - 1) / stride, worst);
+  if (!(worst < 2e-4)) {
+    std::fprintf(stderr, "update differs from the closed form\n");
+    return 4;
+  }
+  hipFree(d_gradient); hipFree(d_update); hipFree(d_copy); hipFree(d_momentum); hipFree(d_variance);
+  hipFree(d_ql); hipFree(d_qr); hipFree(d_workspace);
+  std::printf("ok\n");
+  return 0;
+}
