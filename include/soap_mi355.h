@@ -158,7 +158,10 @@ size_t soapmi_power_iteration_qr_workspace_bytes(int64_t n);
 
 /* refresh_bases_and_transport_optimizer_state_ (src/soap_tp/ops/factorizations.py:550-614):
  * momentum to parameter space with the old bases, power iteration + QR on both sides, variance
- * <- variance[left_order][:, right_order], momentum into the new bases. */
+ * <- variance[left_order][:, right_order], momentum into the new bases.
+ * The two sides' factorisations run side by side: the smaller one is enqueued on a second stream
+ * that the library keeps per device (default priority), forked from `stream` and joined back into
+ * it with events, so for the caller all work is still ordered on `stream`. */
 int soapmi_refresh_f32(float* momentum, int64_t ldm, float* variance, int64_t ldv, float* left_preconditioner,
                        int64_t ldl, float* right_preconditioner, int64_t ldr, float* q_left, int64_t ldql,
                        float* q_right, int64_t ldqr, float* left_work, int64_t ldlw, float* right_work,

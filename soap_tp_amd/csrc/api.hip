@@ -62,6 +62,35 @@ static int resolve_workspace(void* user, size_t user_bytes, size_t need, void** 
   return kOk;
 }
 
+// A second stream per device (default priority) and two events, created on first use and kept
+// for the life of the process: the basis refresh runs its two independent factorisation chains
+// side by side, forked from and joined back into the caller's stream with events, so the caller
+// still sees everything ordered on the stream it passed.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr;
+  hipEvent_t join = nullptr;
+};
+static SideStream g_side[64];
+
+static int side_stream(SideStream** out) {
+  int dev = 0;
+  SOAPMI_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) {
+    set_error("unsupported device index %d", dev);
+    return kRuntimeError;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  SideStream& side = g_side[dev];
+  if (!side.stream) {
+    SOAPMI_HIP(hipStreamCreateWithFlags(&side.stream, hipStreamNonBlocking));
+    SOAPMI_HIP(hipEventCreateWithFlags(&side.fork, hipEventDisableTiming));
+    SOAPMI_HIP(hipEventCreateWithFlags(&side.join, hipEventDisableTiming));
+  }
+  *out = &side;
+  return kOk;
+}
+
 static AdamScalars make_adam_scalars(int64_t step, double beta1, double beta2, double eps_in) {
   AdamScalars s;
   s.beta1 = (float)beta1;
@@ -86,10 +115,6 @@ static int check_adam_args(int64_t step, double beta1, double beta2, double eps)
 
 using namespace soapmi;
 
-static int resolve_workspace_fwd(void* user, size_t user_bytes, size_t need, void** out) {
-  return resolve_workspace(user, user_bytes, need, out);
-}
-
 template <typename T>
 static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_t ldq, void* workspace,
                       size_t workspace_bytes, void* stream) {
@@ -99,7 +124,7 @@ static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_
   SOAPMI_REQUIRE(n <= 32768, "matrix size %lld exceeds the supported maximum 32768", (long long)n);
   const size_t need = eigh_workspace_bytes<T>(n);
   void* ws = nullptr;
-  int rc = resolve_workspace_fwd(workspace, workspace_bytes, need, &ws);
+  int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
   if (rc) return rc;
   Workspace w(ws, need);
   EighWorkspace<T> ews;
@@ -492,12 +517,15 @@ int soapmi_power_iteration_qr_f32(float* p, float* q, float* work, int64_t n, in
 }
 
 size_t soapmi_refresh_workspace_bytes(int64_t rows, int64_t cols) {
-  size_t a = soapmi_rotate_workspace_bytes(rows, cols);
-  size_t b = soapmi_power_iteration_qr_workspace_bytes(rows);
-  size_t c = soapmi_power_iteration_qr_workspace_bytes(cols);
-  size_t d = soapmi_permute_workspace_bytes(rows, cols);
-  size_t m = a > b ? a : b;
-  m = m > c ? m : c;
+  // the two factorisation chains run concurrently and need disjoint scratch; the rotations and
+  // the variance permutation before and after them reuse the same bytes
+  WorkspaceSizer chains;
+  chains.take<char>(soapmi_power_iteration_qr_workspace_bytes(rows));
+  chains.take<char>(soapmi_power_iteration_qr_workspace_bytes(cols));
+  size_t m = chains.total();
+  const size_t a = soapmi_rotate_workspace_bytes(rows, cols);
+  const size_t d = soapmi_permute_workspace_bytes(rows, cols);
+  m = m > a ? m : a;
   return m > d ? m : d;
 }
 
@@ -512,14 +540,36 @@ int soapmi_refresh_f32(float* momentum, int64_t ldm, float* variance, int64_t ld
   void* ws = nullptr;
   int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
   if (rc) return rc;
+  SideStream* side = nullptr;
+  rc = side_stream(&side);
+  if (rc) return rc;
+  hipStream_t main_stream = (hipStream_t)stream;
+  Workspace chains(ws, need);
+  const size_t left_bytes = soapmi_power_iteration_qr_workspace_bytes(rows);
+  const size_t right_bytes = soapmi_power_iteration_qr_workspace_bytes(cols);
+  char* left_ws = chains.take<char>(left_bytes);
+  char* right_ws = chains.take<char>(right_bytes);
+
   rc = soapmi_rotate_f32(q_left, momentum, q_right, rows, cols, ldql, ldm, ldqr, 0, ws, need, stream);
   if (rc) return rc;
-  rc = soapmi_power_iteration_qr_f32(left_preconditioner, q_left, left_work, rows, ldl, ldql, ldlw, symmetrize,
-                                     left_order, nullptr, ws, need, stream);
-  if (rc) return rc;
-  rc = soapmi_power_iteration_qr_f32(right_preconditioner, q_right, right_work, cols, ldr, ldqr, ldrw, symmetrize,
-                                     right_order, nullptr, ws, need, stream);
-  if (rc) return rc;
+  // fork: the smaller chain goes to the side stream, whose latency-bound panel kernels fill the
+  // gaps of the larger one
+  const bool left_on_side = rows <= cols;
+  SOAPMI_HIP(hipEventRecord(side->fork, main_stream));
+  SOAPMI_HIP(hipStreamWaitEvent(side->stream, side->fork, 0));
+  int rc_left = soapmi_power_iteration_qr_f32(left_preconditioner, q_left, left_work, rows, ldl, ldql, ldlw, symmetrize,
+                                              left_order, nullptr, left_ws, left_bytes,
+                                              left_on_side ? (void*)side->stream : stream);
+  int rc_right = kOk;
+  if (rc_left == kOk)
+    rc_right = soapmi_power_iteration_qr_f32(right_preconditioner, q_right, right_work, cols, ldr, ldqr, ldrw,
+                                             symmetrize, right_order, nullptr, right_ws, right_bytes,
+                                             left_on_side ? stream : (void*)side->stream);
+  // join, also after a failure: nothing may stay detached from the caller's stream
+  SOAPMI_HIP(hipEventRecord(side->join, side->stream));
+  SOAPMI_HIP(hipStreamWaitEvent(main_stream, side->join, 0));
+  if (rc_left) return rc_left;
+  if (rc_right) return rc_right;
   rc = soapmi_permute_f32(variance, ldv, rows, cols, left_order, right_order, ws, need, stream);
   if (rc) return rc;
   return soapmi_rotate_f32(q_left, momentum, q_right, rows, cols, ldql, ldm, ldqr, 1, ws, need, stream);
