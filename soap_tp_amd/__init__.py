@@ -6,5 +6,7 @@
 """
 from . import ops
 from .soap import soap_step
+from .optim import SOAP
+from .state_io import load_state, pack_state, save_state, unpack_state, validate_state
 
-__all__ = ["ops", "soap_step"]
+__all__ = ["ops", "soap_step", "SOAP", "save_state", "load_state", "pack_state", "unpack_state", "validate_state"]
