@@ -9,6 +9,8 @@
 // a fixed-order sum over workgroups.  No atomics, so results do not depend on scheduling.
 // Trailing matrix and Q formation: compact-WY block reflectors on the MFMA GEMM.
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 #include "gemm.hpp"
 
@@ -149,45 +151,63 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
 // ---- whole panel in one launch -----------------------------------------------------------------
 // The same column recurrence as qr_panel_step_kernel, but the 32 columns of a panel run inside
 // one launch: every thread keeps its row of the panel in registers from the first column to the
-// last (loaded once, each finished column stored once), and the workgroups meet at a counter in
-// device memory between columns.  Requirements: all workgroups of the launch are resident at the
-// same time (the host launches at most kQrPersistentMaxWg of them, one per CU), and the counter
-// starts the launch at `base`.  Waiting is bounded: a workgroup that does not see the others
-// arrive within kQrSpinLimit polls raises `error` and leaves, and so does everyone who sees the flag.
+// last (loaded once, each finished column stored once).  Between columns the workgroups exchange
+// their partial dot products (and the pivot row) through "mailbox" words in device memory: every
+// value travels as one 64-bit word {float bits, sequence number} written and read with single-copy
+// atomic accesses, so a reader that sees the expected sequence number has the value with it.  No
+// separate flag, counter or fence is needed, and a column costs one trip through memory.
+// Sequence numbers grow by one per column over the whole factorisation (the host passes the
+// launch's starting value and clears the mailboxes before the first panel), mailboxes alternate
+// between two sets by column parity: a workgroup writes column c+2 only after it has read every
+// workgroup's column c+1, which those wrote after they had read column c.
+// Requirements: all workgroups of the launch are resident at the same time (the host launches at
+// most kQrPersistentMaxWg of them, one per CU).  Waiting is bounded: a thread that does not see a
+// word arrive within kQrSpinLimit polls raises `error`, and every workgroup that sees the flag or
+// runs out of patience itself leaves the kernel.
 constexpr int kQrPersistentMaxWg = 128;
 constexpr unsigned kQrSpinLimit = 1u << 22;
 
-__device__ __forceinline__ bool panel_grid_barrier(unsigned* counter, unsigned target, int* error, int* s_fail) {
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    // The release covers this wavefront's own earlier stores, which is why every global value the
-    // other workgroups read after the barrier is written by wavefront 0.
-    __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    int fail = 0;
-    unsigned spins = 0;
-    while (__hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
-      if (++spins > kQrSpinLimit || __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
-        fail = 1;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(2);
-    }
-    if (fail) __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    *s_fail = fail;
-  }
-  __syncthreads();
-  return *s_fail == 0;
+__device__ __forceinline__ unsigned long long mailbox_pack(float value, unsigned seq) {
+  return ((unsigned long long)seq << 32) | (unsigned long long)__float_as_uint(value);
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void qr_panel_persistent_kernel(T* __restrict__ A, int64_t lda, int n, int p, int pe,
-                                                                  T* part, T* piv, T* __restrict__ tau,
-                                                                  unsigned* counter, unsigned base, int* error,
-                                                                  int nwg) {
+// Reads `count` (<= 8) mailbox words until all carry `seq`; false after too many polls or once the
+// error flag is up.
+template <int COUNT>
+__device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&slot)[COUNT], const bool (&used)[COUNT],
+                                             unsigned seq, const int* error, float (&value)[COUNT]) {
+  unsigned spins = 0;
+  for (;;) {
+    unsigned long long word[COUNT];
+#pragma unroll
+    for (int u = 0; u < COUNT; ++u)
+      word[u] = used[u] ? __hip_atomic_load(slot[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                        : mailbox_pack(0.0f, seq);
+    bool ready = true;
+#pragma unroll
+    for (int u = 0; u < COUNT; ++u) ready = ready && (unsigned)(word[u] >> 32) == seq;
+    if (ready) {
+#pragma unroll
+      for (int u = 0; u < COUNT; ++u) value[u] = __uint_as_float((unsigned)word[u]);
+      return true;
+    }
+    ++spins;
+    if (spins > kQrSpinLimit) return false;
+    if ((spins & 63u) == 0 && __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
+__global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restrict__ A, int64_t lda, int n, int p,
+                                                                  int pe, unsigned long long* part,
+                                                                  unsigned long long* piv, float* __restrict__ tau,
+                                                                  unsigned seq_base, int* error, int nwg) {
+  using T = float;
   constexpr int NB = kQrNb;
   __shared__ T s_tc[NB];
   __shared__ T s_wave[4][NB];
   __shared__ T s_sum8[8][NB];
+  __shared__ T s_piv_out[NB];
   __shared__ T s_piv[NB];
   __shared__ T s_scal[3];
   __shared__ int s_fail;
@@ -196,6 +216,7 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(T* __restrict_
   const int r = p + wg * 256 + tid;
   const int nbw = pe - p;
   const bool live = r < n;
+  if (tid == 0) s_fail = 0;
 
   T a[NB];  // a[k] = A[r, j + k] for the current column j: the row is shifted left after each column
 #pragma unroll
@@ -203,8 +224,10 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(T* __restrict_
 
   for (int c = 0; c < nbw; ++c) {
     const int j = p + c;
-    T* part_c = part + (size_t)(c & 1) * nwg * NB;
-    T* piv_c = piv + (c & 1) * NB;
+    const unsigned seq = seq_base + (unsigned)c + 1u;
+    unsigned long long* part_c = part + (size_t)(c & 1) * kQrPersistentMaxWg * NB;
+    unsigned long long* piv_c = piv + (c & 1) * NB;
+    const bool owns_pivot = j >= p + wg * 256 && j < p + wg * 256 + 256;
     // dot products of column j with the remaining panel columns over the rows below the pivot
     {
       const bool below = live && r > j;
@@ -215,35 +238,49 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(T* __restrict_
       if ((lane & 1) == 0) s_wave[wave][(lane >> 1) & 31] = total;
       if (live && r == j) {
 #pragma unroll
-        for (int k = 0; k < NB; ++k) s_piv[k] = a[k];
+        for (int k = 0; k < NB; ++k) s_piv_out[k] = a[k];
       }
     }
     __syncthreads();
     if (tid < NB) {
       const T sum = (s_wave[0][tid] + s_wave[1][tid]) + (s_wave[2][tid] + s_wave[3][tid]);
-      __hip_atomic_store(part_c + wg * NB + tid, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (j >= p + wg * 256 && j < p + wg * 256 + 256)  // this workgroup owns the pivot row
-        __hip_atomic_store(piv_c + tid, s_piv[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(part_c + wg * NB + tid, mailbox_pack(sum, seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (owns_pivot)
+        __hip_atomic_store(piv_c + tid, mailbox_pack(s_piv_out[tid], seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (!panel_grid_barrier(counter, base + (unsigned)nwg * (unsigned)(c + 1), error, &s_fail)) return;
     {
       // fixed-order sum of the per-workgroup partials, as in qr_panel_step_kernel
       const int k = tid & (NB - 1), g = tid >> 5;
       T s = T(0);
-      for (int w0 = g; w0 < nwg; w0 += 64) {
-        T v[8];
+      bool ok = true;
+      for (int w0 = g; w0 < nwg && ok; w0 += 64) {
+        const unsigned long long* slot[8];
+        bool used[8];
+        float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          v[u] = (w0 + 8 * u < nwg)
-                     ? __hip_atomic_load(part_c + (w0 + 8 * u) * NB + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                     : T(0);
+        for (int u = 0; u < 8; ++u) {
+          used[u] = w0 + 8 * u < nwg;
+          slot[u] = part_c + (used[u] ? (w0 + 8 * u) : 0) * NB + k;
+        }
+        ok = mailbox_wait<8>(slot, used, seq, error, v);
 #pragma unroll
         for (int u = 0; u < 8; ++u) s += v[u];
       }
       s_sum8[g][k] = s;
-      if (tid < NB) s_piv[tid] = __hip_atomic_load(piv_c + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid < NB && ok) {
+        const unsigned long long* slot[1] = {piv_c + tid};
+        const bool used[1] = {true};
+        float v[1];
+        ok = mailbox_wait<1>(slot, used, seq, error, v);
+        s_piv[tid] = v[0];
+      }
+      if (!ok) {
+        __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_fail = 1;
+      }
     }
     __syncthreads();
+    if (s_fail) return;
     if (tid < NB) {
       T x2 = T(0), dot = T(0);
 #pragma unroll
@@ -283,8 +320,9 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(T* __restrict_
 #pragma unroll
     for (int k = 0; k + 1 < NB; ++k) a[k] = a[k + 1];
     a[NB - 1] = T(0);
-    // s_piv, s_wave are rewritten only after the next __syncthreads pair; s_tc is read above
-    __syncthreads();
+    // No barrier here: the shared arrays of the next column's first phase (s_wave, s_piv_out) were
+    // last read before the barrier that follows the mailbox phase, and s_tc / s_scal are rewritten
+    // only behind the next such barrier, which every wavefront reaches after this point.
   }
 }
 
@@ -496,12 +534,13 @@ static inline void launch_extract_v(hipStream_t s, const T* A, int64_t lda, int 
 template <typename T>
 struct QrWorkspace {
   BlockReflectorWs<T> br;
-  T* t_in;    // kBrMax x kBrMax   factor of the current inner panel
   T* t_all;   // outer blocks x kBrMax x kBrMax
   T* tau;     // n
-  T* part;    // 2 x nwg x NB
+  T* part;    // 2 x nwg x NB   partials of the launch-per-column fallback
   T* piv;     // 2 x NB
-  unsigned* sync;  // [0] arrival counter of the persistent panel kernel, [1] its error flag
+  unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x NB   mailboxes of the persistent panel kernel
+  unsigned long long* mail_piv;   // 2 x NB
+  unsigned* sync;  // [1] error flag of the persistent panel kernel
 };
 
 template <typename T, class WS>
@@ -510,11 +549,12 @@ static inline void qr_workspace_layout(WS& ws, int64_t n, QrWorkspace<T>* out) {
   const int64_t blocks = ceil_div64(n, kBrMax);
   const int64_t nwg = ceil_div64(n, 256);
   block_reflector_layout<T>(ws, n, out ? &q.br : nullptr);
-  q.t_in = ws.template take<T>(kBrMax * kBrMax);
   q.t_all = ws.template take<T>((size_t)blocks * kBrMax * kBrMax);
   q.tau = ws.template take<T>((size_t)n);
   q.part = ws.template take<T>((size_t)2 * nwg * kQrNb);
   q.piv = ws.template take<T>(2 * kQrNb);
+  q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * kQrNb);
+  q.mail_piv = ws.template take<unsigned long long>(2 * kQrNb);
   q.sync = ws.template take<unsigned>(64);
   if (out) *out = q;
 }
@@ -537,8 +577,15 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
   int rc;
-  unsigned sync_base = 0;
+  static_assert(std::is_same<T, float>::value, "the persistent panel kernel packs float values into its mailboxes");
+  unsigned seq_base = 0;
   hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
+  {
+    // mail_part and mail_piv are adjacent: one clear covers both (sequence number 0 = "nothing yet")
+    const int words = 2 * (2 * kQrPersistentMaxWg * kQrNb + 2 * kQrNb);
+    hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3((words + 255) / 256), dim3(256), 0, s,
+                       reinterpret_cast<unsigned*>(ws.mail_part), words);
+  }
   // ---- factorisation ----
   for (int bi = 0; bi < blocks; ++bi) {
     const int P = bi * OB, PE = std::min(n, P + OB), obw = PE - P;
@@ -552,9 +599,9 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
       T* piv[2] = {ws.piv, ws.piv + NB};
       if (nwg <= kQrPersistentMaxWg) {
-        hipLaunchKernelGGL((qr_panel_persistent_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.part,
-                           ws.piv, ws.tau, ws.sync, sync_base, reinterpret_cast<int*>(ws.sync + 1), nwg);
-        sync_base += (unsigned)nwg * (unsigned)nbw;
+        hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
+                           ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg);
+        seq_base += (unsigned)nbw;
       } else {
         for (int j = p - 1; j < pe; ++j) {
           const int in = (j - p + 1) & 1, out = in ^ 1;
