@@ -48,11 +48,6 @@ template <typename T>
 static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, int64_t ldz, int n,
                                  const EighWorkspace<T>& ws) {
   if (n <= 0) return kOk;
-  {
-    const unsigned nb = (unsigned)ceil_div64(n, 64);
-    hipLaunchKernelGGL((symmetrize_lower_kernel<T>), dim3(nb, nb), dim3(256), 0, s, A, lda, n);
-    SOAPMI_LAUNCH_CHECK();
-  }
   int rc = sytrd_lower<T>(s, A, lda, n, ws.d, ws.e, ws.tau, ws.trd);
   if (rc) return rc;
   rc = stedc<T>(s, n, ws.d, ws.e, w, Z, ldz, ws.dc);

@@ -503,4 +503,15 @@ static inline int gemm(hipStream_t stream, int transA, int transB, int M, int N,
   return launch_gemm<T, EpiStore<T>, Cfg>(stream, p, ep, 1);
 }
 
+// Square product restricted to the tiles on or below the diagonal of C (n x n): entries of C above
+// the diagonal tiles are neither read nor written; inside diagonal tiles the whole tile is updated.
+template <typename T, class Cfg = typename DefaultTile<T>::type>
+static inline int gemm_lower(hipStream_t stream, int transA, int transB, int n, int K, T alpha, const T* A,
+                             int64_t lda, const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {
+  if (n <= 0) return kOk;
+  GemmProblem<T> p = make_problem<T, Cfg>(transA, transB, n, n, K, A, lda, B, ldb, true);
+  EpiStore<T> ep{C, ldc, alpha, beta};
+  return launch_gemm<T, EpiStore<T>, Cfg>(stream, p, ep, 1);
+}
+
 }  // namespace soapmi

@@ -31,12 +31,52 @@ __device__ __forceinline__ void butterfly_stage(T (&vals)[32], int lane) {
   }
 }
 
+// The two widest stages (partners 32 and 16 lanes apart) on gfx950's lane-swap instructions:
+// v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second
+// (v_permlane16_swap: the odd 16-lane rows of the first with the even rows of the second), which is
+// exactly "send the half I do not keep, receive the half I keep": afterwards the two registers hold
+// the two addends in every lane, with no select and no trip through the LDS crossbar.
+template <bool WIDE32>
+__device__ __forceinline__ void lane_swap(unsigned& a, unsigned& b) {
+  if constexpr (WIDE32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    a = r[0];
+    b = r[1];
+  } else {
+    const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+    a = r[0];
+    b = r[1];
+  }
+}
+
+template <bool WIDE32>
+__device__ __forceinline__ float swap_add(float a, float b) {
+  unsigned ua = __float_as_uint(a), ub = __float_as_uint(b);
+  lane_swap<WIDE32>(ua, ub);
+  return __uint_as_float(ua) + __uint_as_float(ub);
+}
+
+template <bool WIDE32>
+__device__ __forceinline__ double swap_add(double a, double b) {
+  unsigned a_lo = (unsigned)__double2loint(a), a_hi = (unsigned)__double2hiint(a);
+  unsigned b_lo = (unsigned)__double2loint(b), b_hi = (unsigned)__double2hiint(b);
+  lane_swap<WIDE32>(a_lo, b_lo);
+  lane_swap<WIDE32>(a_hi, b_hi);
+  return __hiloint2double((int)a_hi, (int)a_lo) + __hiloint2double((int)b_hi, (int)b_lo);
+}
+
+template <typename T, int HALF, bool WIDE32>
+__device__ __forceinline__ void butterfly_stage_swap(T (&vals)[32]) {
+#pragma unroll
+  for (int c = 0; c < HALF; ++c) vals[c] = swap_add<WIDE32>(vals[c], vals[c + HALF]);
+}
+
 // After the call lane l holds, in the return value, the sum over the wavefront of vals[(l>>1)&31].
 // Stages are spelled out so that every register index is a compile-time constant.
 template <typename T>
 __device__ __forceinline__ T wave_reduce_32(T (&vals)[32], int lane) {
-  butterfly_stage<T, 16, 32>(vals, lane);
-  butterfly_stage<T, 8, 16>(vals, lane);
+  butterfly_stage_swap<T, 16, true>(vals);
+  butterfly_stage_swap<T, 8, false>(vals);
   butterfly_stage<T, 4, 8>(vals, lane);
   butterfly_stage<T, 2, 4>(vals, lane);
   butterfly_stage<T, 1, 2>(vals, lane);

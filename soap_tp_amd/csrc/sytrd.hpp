@@ -7,11 +7,13 @@
 //      rank-2 updates, partial sums of the sub-column norm
 //   B  reflector scalars (every workgroup re-derives them from the same partial sums), v, and
 //      partial products W^T v, V^T v
-//   C  y = A_trailing v : the bandwidth-bound kernel; a workgroup owns 256 rows x one column chunk,
-//      lanes run along rows so every load instruction reads 512 contiguous bytes
+//   C  y = A_trailing v : the bandwidth-bound kernel.  Only the lower triangle is read: a workgroup
+//      owns one 128 x 128 tile on or below the diagonal and produces both the tile's product with
+//      v (for its rows) and the transposed tile's product (for its columns, a wavefront butterfly
+//      per 32 columns); lanes run along rows so every load instruction reads 512 contiguous bytes
 //   D  w = tau (y - V (W^T v) - W (V^T v)) and partial sums of w^T v
-// The trailing matrix keeps both triangles valid (the rank-2k update runs on the MFMA GEMM over
-// the full square), so kernel C is a plain column-major matrix-vector product.
+// The rank-2k update of the trailing matrix runs on the MFMA product over the tiles on or below
+// the diagonal only, as one product with K = 64: A -= [V | W] [W | V]^T.
 // All cross-workgroup reductions are "write partials, every consumer re-sums them in the same
 // order": no atomics, reproducible results.
 #pragma once
@@ -22,13 +24,14 @@
 namespace soapmi {
 
 constexpr int kTrdNb = 32;        // panel width
-constexpr int kTrdMaxChunks = 32; // column chunks of the matrix-vector product
+constexpr int kTrdTile = 128;     // tile edge of the matrix-vector product
 
 template <typename T>
 struct TrdWorkspace {
   T* vc;        // n x NB   clean reflector block of the current panel (rows are global indices)
-  T* w;         // n x NB
-  T* y_part;    // kTrdMaxChunks x n
+  T* w;         // n x NB   directly behind vc: [vc | w] is one n x 2NB operand
+  T* vc2;       // n x NB   copy of vc directly behind w: [w | vc2] is the other operand
+  T* y_part;    // ceil(n / kTrdTile) x n   one slot per tile that touches an index
   T* norm_part; // nwg
   T* dot_part;  // nwg
   T* t_part;    // nwg x 2*NB   partial (W^T v | V^T v)
@@ -39,14 +42,16 @@ struct TrdWorkspace {
 template <typename T, class WS>
 static inline void trd_workspace_layout(WS& ws, int64_t n, TrdWorkspace<T>* out) {
   const int64_t nwg = ceil_div64(n, 256);
-  T* vc = ws.template take<T>((size_t)n * kTrdNb);
-  T* w = ws.template take<T>((size_t)n * kTrdNb);
-  T* y_part = ws.template take<T>((size_t)n * kTrdMaxChunks);
+  // one allocation, so that the three blocks are adjacent whatever the allocator's alignment is
+  T* vc = ws.template take<T>((size_t)3 * n * kTrdNb);
+  T* w = vc + (size_t)n * kTrdNb;
+  T* vc2 = w + (size_t)n * kTrdNb;
+  T* y_part = ws.template take<T>((size_t)n * ceil_div64(n, kTrdTile));
   T* norm_part = ws.template take<T>((size_t)nwg);
   T* dot_part = ws.template take<T>((size_t)nwg);
   T* t_part = ws.template take<T>((size_t)nwg * 2 * kTrdNb);
   T* scal = ws.template take<T>(16);
-  if (out) *out = TrdWorkspace<T>{vc, w, y_part, norm_part, dot_part, t_part, scal, (int)nwg};
+  if (out) *out = TrdWorkspace<T>{vc, w, vc2, y_part, norm_part, dot_part, t_part, scal, (int)nwg};
 }
 
 template <typename T>
@@ -151,7 +156,8 @@ __global__ __launch_bounds__(256) void trd_finish_w_kernel(T* __restrict__ W, co
 // Kernel B.  Rows r >= j+1 (workgroup/thread mapping: r = j + 1 + ...).
 template <typename T>
 __global__ __launch_bounds__(256) void trd_reflector_kernel(T* __restrict__ A, int64_t lda, int n, int p, int j,
-                                                            T* __restrict__ Vc, const T* __restrict__ W, int64_t ldw,
+                                                            T* __restrict__ Vc, T* __restrict__ Vc2,
+                                                            const T* __restrict__ W, int64_t ldw,
                                                             const T* __restrict__ norm_part, int n_norm_part,
                                                             T* __restrict__ tau, T* __restrict__ e,
                                                             T* __restrict__ t_part) {
@@ -189,10 +195,14 @@ __global__ __launch_bounds__(256) void trd_reflector_kernel(T* __restrict__ A, i
       A[r + (int64_t)j * lda] = v;  // reflector kept for the back-transformation
     }
     Vc[r + (int64_t)i * ldw] = v;
+    Vc2[r + (int64_t)i * ldw] = v;
   }
   // rows <= j of this column of Vc must read as zero for later row-j lookups
   if (blockIdx.x == 0) {
-    for (int rr = p + tid; rr <= j; rr += 256) Vc[rr + (int64_t)i * ldw] = T(0);
+    for (int rr = p + tid; rr <= j; rr += 256) {
+      Vc[rr + (int64_t)i * ldw] = T(0);
+      Vc2[rr + (int64_t)i * ldw] = T(0);
+    }
   }
   // partial W^T v and V^T v over this workgroup's rows (columns k < i): 2*NB products per thread,
   // two 32-value butterflies per wavefront
@@ -220,39 +230,76 @@ __global__ __launch_bounds__(256) void trd_reflector_kernel(T* __restrict__ A, i
   }
 }
 
-// Kernel C.  y_part[chunk][r] = sum over this chunk's columns of A[r, c] v[c];  rows and columns
-// both run over j+1 .. n-1.  v is read from column i of Vc.
+// Kernel C.  The trailing matrix (rows and columns o = j+1 .. n-1, only its lower triangle is
+// valid) is cut into 128 x 128 tiles from its own origin; workgroup t owns tile (rb, cb), cb <= rb.
+// 256 threads: thread (row = tid % 128, half = tid / 128) holds 64 entries of its row.  It adds
+// a[row, c] v[c] to the row's sum ("direct") and, for the mirrored upper triangle, contributes
+// a[row, c] v[row] to column c's sum, reduced over the rows by wavefront butterflies.
+// y_part has one slot per tile edge: index i of block b receives slot s < b from tile (b, s)'s direct
+// sums, slot s > b from tile (s, b)'s column sums, and slot b from the diagonal tile, which adds
+// both.  Every (slot, index) pair is written exactly once, so kernel D sums nb slots per index in a
+// fixed order and nothing has to be cleared.
 template <typename T>
 __global__ __launch_bounds__(256) void trd_symv_kernel(const T* __restrict__ A, int64_t lda, int n, int j,
-                                                       const T* __restrict__ v, T* __restrict__ y_part, int chunk_w) {
-  __shared__ T s_v[512];
-  const int tid = threadIdx.x;
-  const int r = j + 1 + blockIdx.x * 256 + tid;
-  const int c_begin = j + 1 + blockIdx.y * chunk_w;
-  const int c_end = min(n, c_begin + chunk_w);
-  T acc0 = T(0), acc1 = T(0), acc2 = T(0), acc3 = T(0);
-  for (int cb = c_begin; cb < c_end; cb += 512) {
-    const int cnt = min(512, c_end - cb);
-    __syncthreads();
-    for (int t = tid; t < cnt; t += 256) s_v[t] = v[cb + t];
-    __syncthreads();
-    if (r < n) {
-      const T* col = A + r + (int64_t)cb * lda;
-      int c = 0;
-      for (; c + 4 <= cnt; c += 4) {
-        const T a0 = col[(int64_t)(c + 0) * lda];
-        const T a1 = col[(int64_t)(c + 1) * lda];
-        const T a2 = col[(int64_t)(c + 2) * lda];
-        const T a3 = col[(int64_t)(c + 3) * lda];
-        acc0 += a0 * s_v[c + 0];
-        acc1 += a1 * s_v[c + 1];
-        acc2 += a2 * s_v[c + 2];
-        acc3 += a3 * s_v[c + 3];
-      }
-      for (; c < cnt; ++c) acc0 += col[(int64_t)c * lda] * s_v[c];
+                                                       const T* __restrict__ v, T* __restrict__ y_part) {
+  constexpr int TS = kTrdTile;
+  __shared__ T s_v[TS];
+  __shared__ T s_direct[2][TS];
+  __shared__ T s_col[4][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // `half` is the same for all lanes of a wavefront: telling the compiler so moves the column
+  // address arithmetic to the scalar unit
+  const int row = tid & (TS - 1), half = __builtin_amdgcn_readfirstlane(tid >> 7);
+  const int o = j + 1;
+  const int t = blockIdx.x;
+  int rb = (int)((sqrtf(8.0f * (float)t + 1.0f) - 1.0f) * 0.5f);
+  while (rb * (rb + 1) / 2 > t) --rb;
+  while ((rb + 1) * (rb + 2) / 2 <= t) ++rb;
+  const int cb = t - rb * (rb + 1) / 2;
+  const int r = o + rb * TS + row;        // global row of this thread
+  const int c0 = o + cb * TS;             // first global column of the tile
+  const bool live = r < n;
+  const bool diagonal = rb == cb;
+  if (tid < TS) s_v[tid] = (c0 + tid < n) ? v[c0 + tid] : T(0);
+  const T vr = live ? v[r] : T(0);
+  __syncthreads();
+  T acc0 = T(0), acc1 = T(0);
+  // Loads are unconditional on clamped addresses (always inside the matrix); what must not count
+  // - rows past the end, the upper triangle inside a diagonal tile - is zeroed after the load.
+  const int rr = min(r, n - 1);
+  const int limit = diagonal ? r : n - 1;  // last column that counts for this row
+#pragma unroll 1
+  for (int q = 0; q < 2; ++q) {  // 32 columns at a time
+    const int cq = c0 + 64 * half + 32 * q;
+    T a[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) a[k] = A[rr + (int64_t)min(cq + k, n - 1) * lda];
+    T cols[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      const T x = (live && cq + k <= limit) ? a[k] : T(0);
+      if (k & 1) acc1 += x * s_v[64 * half + 32 * q + k];
+      else acc0 += x * s_v[64 * half + 32 * q + k];
+      cols[k] = (diagonal && cq + k == r) ? T(0) : x * vr;  // the diagonal entry counts once
+    }
+    const T total = wave_reduce_32<T>(cols, lane);
+    if ((lane & 1) == 0) s_col[wave][32 * q + ((lane >> 1) & 31)] = total;
+  }
+  s_direct[half][row] = acc0 + acc1;
+  __syncthreads();
+  if (tid < TS) {
+    // wavefronts 2*half and 2*half+1 hold the two row halves of column half `half`
+    const int h = tid >> 6, k = tid & 63;
+    const T column_sum = s_col[2 * h][k] + s_col[2 * h + 1][k];
+    const T row_sum = s_direct[0][tid] + s_direct[1][tid];
+    const int gr = o + rb * TS + tid, gc = c0 + tid;
+    if (diagonal) {
+      if (gr < n) y_part[(int64_t)rb * n + gr] = row_sum + column_sum;
+    } else {
+      if (gr < n) y_part[(int64_t)cb * n + gr] = row_sum;
+      if (gc < n) y_part[(int64_t)rb * n + gc] = column_sum;
     }
   }
-  if (r < n) y_part[(int64_t)blockIdx.y * n + r] = (acc0 + acc1) + (acc2 + acc3);
 }
 
 // Kernel D.  Rows r >= j+1.
@@ -281,17 +328,20 @@ __global__ __launch_bounds__(256) void trd_w_kernel(int n, int p, int j, const T
   __syncthreads();
   T prod = T(0);
   if (r < n) {
-    T yp[kTrdMaxChunks], wr[NB], vr[NB];
-#pragma unroll
-    for (int c = 0; c < kTrdMaxChunks; ++c) yp[c] = (c < n_chunks) ? y_part[(int64_t)c * n + r] : T(0);
+    T wr[NB], vr[NB];
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
       vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
       wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
     }
     T y = T(0);
+    for (int c0 = 0; c0 < n_chunks; c0 += 16) {  // 16 slot loads in flight, summed in slot order
+      T yp[16];
 #pragma unroll
-    for (int c = 0; c < kTrdMaxChunks; ++c) y += yp[c];
+      for (int c = 0; c < 16; ++c) yp[c] = (c0 + c < n_chunks) ? y_part[(int64_t)(c0 + c) * n + r] : T(0);
+#pragma unroll
+      for (int c = 0; c < 16; ++c) y += yp[c];
+    }
     T corr = T(0);
 #pragma unroll
     for (int k = 0; k < NB; ++k) corr += vr[k] * s_t[k] + wr[k] * s_t[NB + k];
@@ -304,7 +354,7 @@ __global__ __launch_bounds__(256) void trd_w_kernel(int n, int p, int j, const T
 }
 
 // d[n-1] after all updates: the last column has no reflector of its own.
-// Tridiagonalise A (n x n, both triangles valid on entry; destroyed).  On exit d[0..n), e[0..n-1),
+// Tridiagonalise A (n x n, lower triangle referenced; destroyed).  On exit d[0..n), e[0..n-1),
 // tau[0..n-1) and, below the first subdiagonal of A, the reflector vectors (implicit unit at
 // row j+1 of column j), as LAPACK sytrd('L') leaves them.
 template <typename T>
@@ -327,14 +377,12 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
       if (j == n - 1) break;  // only the diagonal entry remained
       const int nt = n - j - 1;
       const int nwgB = (int)ceil_div64(nt, 256);
-      hipLaunchKernelGGL((trd_reflector_kernel<T>), dim3(nwgB), dim3(256), 0, s, A, lda, n, p, j, ws.vc, ws.w, ldw,
-                         ws.norm_part, nwgA, tau, e, ws.t_part);
-      int chunks = (int)std::min<int64_t>(kTrdMaxChunks, ceil_div64(nt, 64));
-      const int chunk_w = (int)ceil_div64(nt, chunks);
-      chunks = (int)ceil_div64(nt, chunk_w);
-      hipLaunchKernelGGL((trd_symv_kernel<T>), dim3(nwgB, chunks), dim3(256), 0, s, A, lda, n, j,
-                         ws.vc + (int64_t)i * ldw, ws.y_part, chunk_w);
-      hipLaunchKernelGGL((trd_w_kernel<T>), dim3(nwgB), dim3(256), 0, s, n, p, j, ws.vc, ws.w, ldw, ws.y_part, chunks,
+      hipLaunchKernelGGL((trd_reflector_kernel<T>), dim3(nwgB), dim3(256), 0, s, A, lda, n, p, j, ws.vc, ws.vc2, ws.w,
+                         ldw, ws.norm_part, nwgA, tau, e, ws.t_part);
+      const int nb = (int)ceil_div64(nt, kTrdTile);
+      hipLaunchKernelGGL((trd_symv_kernel<T>), dim3(nb * (nb + 1) / 2), dim3(256), 0, s, A, lda, n, j,
+                         ws.vc + (int64_t)i * ldw, ws.y_part);
+      hipLaunchKernelGGL((trd_w_kernel<T>), dim3(nwgB), dim3(256), 0, s, n, p, j, ws.vc, ws.w, ldw, ws.y_part, nb,
                          ws.t_part, nwgB, tau, ws.dot_part);
       last_dot_parts = nwgB;
       cols_done = i + 1;
@@ -347,12 +395,20 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
                        ldw, n, pe, cols_done - 1, ws.dot_part, last_dot_parts, tau + jl);
     last_dot_parts = 0;
     const int nt = n - pe;
-    int rc = gemm<T>(s, 0, 1, nt, nt, cols_done, T(-1), ws.vc + pe, ldw, ws.w + pe, ldw, T(1),
-                     A + pe + (int64_t)pe * lda, lda);
-    if (rc) return rc;
-    rc = gemm<T>(s, 0, 1, nt, nt, cols_done, T(-1), ws.w + pe, ldw, ws.vc + pe, ldw, T(1), A + pe + (int64_t)pe * lda,
-                 lda);
-    if (rc) return rc;
+    // A[pe:, pe:] -= [V | W] [W | V]^T, tiles on or below the diagonal only
+    int rc;
+    if (cols_done == NB) {
+      rc = gemm_lower<T>(s, 0, 1, nt, 2 * NB, T(-1), ws.vc + pe, ldw, ws.w + pe, ldw, T(1), A + pe + (int64_t)pe * lda,
+                         lda);
+      if (rc) return rc;
+    } else {
+      rc = gemm_lower<T>(s, 0, 1, nt, cols_done, T(-1), ws.vc + pe, ldw, ws.w + pe, ldw, T(1),
+                         A + pe + (int64_t)pe * lda, lda);
+      if (rc) return rc;
+      rc = gemm_lower<T>(s, 0, 1, nt, cols_done, T(-1), ws.w + pe, ldw, ws.vc + pe, ldw, T(1),
+                         A + pe + (int64_t)pe * lda, lda);
+      if (rc) return rc;
+    }
   }
   return kOk;
 }
