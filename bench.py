@@ -130,7 +130,7 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True):
     return result
 
 
-def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True):
+def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True, full_init=False):
     """The CPU oracle on a bounded sample: `sample_plain_steps` steady-state steps and one refresh."""
     from oracle import soap_oracle as oracle
 
@@ -159,15 +159,66 @@ def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True):
         start = time.perf_counter()
         oracle.refresh(state)
         refresh_ms = (time.perf_counter() - start) * 1e3
+    # one of the two eigensolves of the initialising call (the smaller side, fp64 solve of -P as the
+    # "elpa" variant does); the larger side only on request, it takes most of a minute
+    init_sizes = [min(rows, columns)] + ([max(rows, columns)] if full_init and rows != columns else [])
+    init_ms = {}
+    for size in init_sizes:
+        matrix = state["left_preconditioner"] if size == rows else state["right_preconditioner"]
+        start = time.perf_counter()
+        oracle.eigh_descending(matrix, "elpa")
+        init_ms[str(size)] = (time.perf_counter() - start) * 1e3
     interval = HYPER["basis_refresh_interval"]
     per_step_ms = plain_ms + (refresh_ms / interval if refresh_ms is not None else 0.0)
     return {
         "value": 1e3 / per_step_ms, "unit": "steps/s", "cores": cores, "kind": "port",
         "sample": f"{sample_plain_steps} steady-state steps" + (" + 1 basis refresh" if with_refresh else "")
                   + f" of the {rows}x{columns} workload on the CPU oracle (torch/MKL), refresh cost spread over "
-                  + f"{interval} steps",
-        "plain_step_ms": plain_ms, "refresh_ms": refresh_ms,
+                  + f"{interval} steps; plus the initialising fp64 eigensolve of size(s) {', '.join(init_ms)} "
+                  + "(reported, not part of value)",
+        "plain_step_ms": plain_ms, "refresh_ms": refresh_ms, "init_eigensolve_ms_by_size": init_ms,
     }
+
+
+def run_layer(device, steps=30, rank=64):
+    """One transformer layer's seven matrices (q, k, v, o, gate, up, down), each with its own state,
+    stepped together by the optimizer wrapper: whole-layer time per optimizer step."""
+    from soap_tp_amd import SOAP
+
+    shapes = [(4096, 4096)] * 4 + [(4096, 14336)] * 2 + [(14336, 4096)]
+    parameters = [torch.nn.Parameter(torch.zeros(shape, device=device)) for shape in shapes]
+    gradients = {shape: [device_low_rank_plus_noise(shape[0], shape[1], rank, 42 + 1000 * i + t, device)
+                         for t in range(2)] for i, shape in enumerate(dict.fromkeys(shapes))}
+    optimizer = SOAP(parameters, lr=3e-3, betas=(HYPER["beta1"], HYPER["beta2"]),
+                     shampoo_beta=HYPER["preconditioner_beta"], eps=HYPER["eps"], weight_decay=0.0,
+                     precondition_frequency=HYPER["basis_refresh_interval"])
+
+    def one_step(t):
+        for parameter in parameters:
+            parameter.grad = gradients[tuple(parameter.shape)][t % 2]
+        optimizer.step()
+
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    one_step(0)
+    torch.cuda.synchronize()
+    init_ms = (time.perf_counter() - start) * 1e3
+    interval = HYPER["basis_refresh_interval"]
+    for t in range(1, interval + 1):  # up to and including the first refresh
+        one_step(t)
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record()
+    for t in range(steps):
+        one_step(interval + 1 + t)
+    end.record()
+    torch.cuda.synchronize()
+    total_ms = begin.elapsed_time(end)
+    flops = sum(5.0 * m * n * (m + n) for m, n in shapes)
+    return {"workload": "4 x 4096x4096, 2 x 4096x14336, 1 x 14336x4096, rank 64, refresh every 10, "
+                        "optimizer wrapper with 2 side streams", "steps": steps,
+            "ms_per_layer_step": total_ms / steps, "layer_steps_per_s": steps / (total_ms * 1e-3),
+            "initialisation_ms": init_ms, "plain_step_mfma_flops": flops}
 
 
 def calibration_copies(rows, columns, count, device):
@@ -194,6 +245,11 @@ def main():
     parser.add_argument("--rank", type=int, default=128)
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-other-shapes", action="store_true")
+    parser.add_argument("--cpu-full-init", action="store_true",
+                        help="also time the larger side's initialising eigensolve on the CPU oracle (about a minute)")
+    parser.add_argument("--layer", action="store_true",
+                        help="also run the whole-layer configuration (4 x 4096x4096, 2 x 4096x14336, 1 x 14336x4096, "
+                             "rank 64, 30 steps) through the optimizer wrapper and report it under 'layer'")
     parser.add_argument("--calibration-copies", type=int, default=0,
                         help="run this many layout copies of one rows x columns fp32 matrix (transpose_kernel: "
                              "4*rows*columns bytes read and as many written) before the schedule; the known-size "
@@ -276,8 +332,10 @@ def main():
                 "initialisation_call_ms": run["init_ms"], "step_mfma_stages_tflops": flops / (plain * 1e-3) / 1e12,
             }
         line["other_shapes"] = others
+    if args.layer:
+        line["layer"] = run_layer(device)
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.shape, args.rank)
+        line["cpu_baseline"] = cpu_baseline(args.shape, args.rank, full_init=args.cpu_full_init)
     else:
         line["cpu_baseline"] = None
     print(json.dumps(line))
