@@ -2,20 +2,24 @@
 // lower storage), the first stage of the eigensolver that replaces ELPA's one-stage solver
 // (src/soap_tp/csrc/elpa_bindings.cpp:149,165).
 //
-// Per column j of a panel four launches run, each ending where a matrix-wide reduction is needed:
-//   A  finish the previous w (w += alpha2 v), bring column j up to date with the panel's pending
-//      rank-2 updates, partial sums of the sub-column norm
-//   B  reflector scalars (every workgroup re-derives them from the same partial sums), v, and
-//      partial products W^T v, V^T v
-//   C  y = A_trailing v : the bandwidth-bound kernel.  Only the lower triangle is read: a workgroup
+// Per column j of a panel the work falls into four steps, separated by matrix-wide reductions:
+//   A  bring column j up to date with the panel's pending rank-2 updates (after finishing the
+//      previous w: w += alpha2 v), partial sums of the sub-column norm
+//   B  reflector scalars, v, and partial products W^T v, V^T v
+//   C  y = A_trailing v : the bandwidth-bound step.  Only the lower triangle is read: a workgroup
 //      owns one 128 x 128 tile on or below the diagonal and produces both the tile's product with
 //      v (for its rows) and the transposed tile's product (for its columns, a wavefront butterfly
 //      per 32 columns); lanes run along rows so every load instruction reads 512 contiguous bytes
 //   D  w = tau (y - V (W^T v) - W (V^T v)) and partial sums of w^T v
+// Two launches per column: C (trd_symv_kernel, the whole chip) and one fused kernel that runs
+// D(j), A(j+1), B(j+1) with a thread per row that keeps its rows of V and W in registers across the
+// three steps.  The two reductions inside the fused kernel (w^T v, the norm) travel between its
+// workgroups (at most 128, one per 256 rows) as sequence-tagged 64-bit words in device memory,
+// like the partial sums of the QR panel kernel; the other reductions cross a launch boundary as
+// "write per-workgroup partials, every consumer re-sums them in the same order".  No atomics on
+// data, reproducible results.
 // The rank-2k update of the trailing matrix runs on the MFMA product over the tiles on or below
 // the diagonal only, as one product with K = 64: A -= [V | W] [W | V]^T.
-// All cross-workgroup reductions are "write partials, every consumer re-sums them in the same
-// order": no atomics, reproducible results.
 #pragma once
 #include "common.hpp"
 #include "gemm.hpp"
@@ -25,6 +29,7 @@ namespace soapmi {
 
 constexpr int kTrdNb = 32;        // panel width
 constexpr int kTrdTile = 128;     // tile edge of the matrix-vector product
+constexpr int kTrdMaxWg = 128;    // workgroups of the fused column kernel (256 rows each)
 
 template <typename T>
 struct TrdWorkspace {
@@ -32,11 +37,10 @@ struct TrdWorkspace {
   T* w;         // n x NB   directly behind vc: [vc | w] is one n x 2NB operand
   T* vc2;       // n x NB   copy of vc directly behind w: [w | vc2] is the other operand
   T* y_part;    // ceil(n / kTrdTile) x n   one slot per tile that touches an index
-  T* norm_part; // nwg
   T* dot_part;  // nwg
   T* t_part;    // nwg x 2*NB   partial (W^T v | V^T v)
-  T* scal;      // small: [0] tau_j  [1] alpha2 (unused slots spare)
-  int nwg;
+  unsigned long long* mail;  // 2 reductions x (kTrdMaxWg + 1) values x 2 words
+  int* error;   // raised by a workgroup that gave up waiting for a message
 };
 
 template <typename T, class WS>
@@ -47,11 +51,11 @@ static inline void trd_workspace_layout(WS& ws, int64_t n, TrdWorkspace<T>* out)
   T* w = vc + (size_t)n * kTrdNb;
   T* vc2 = w + (size_t)n * kTrdNb;
   T* y_part = ws.template take<T>((size_t)n * ceil_div64(n, kTrdTile));
-  T* norm_part = ws.template take<T>((size_t)nwg);
   T* dot_part = ws.template take<T>((size_t)nwg);
   T* t_part = ws.template take<T>((size_t)nwg * 2 * kTrdNb);
-  T* scal = ws.template take<T>(16);
-  if (out) *out = TrdWorkspace<T>{vc, w, vc2, y_part, norm_part, dot_part, t_part, scal, (int)nwg};
+  unsigned long long* mail = ws.template take<unsigned long long>(2 * (kTrdMaxWg + 1) * 2 + 2);
+  int* error = reinterpret_cast<int*>(mail + 2 * (kTrdMaxWg + 1) * 2);
+  if (out) *out = TrdWorkspace<T>{vc, w, vc2, y_part, dot_part, t_part, mail, error};
 }
 
 template <typename T>
@@ -77,71 +81,79 @@ __device__ __forceinline__ T reduce_partials(const T* __restrict__ part, int cou
   return block_sum_256(s, red);
 }
 
-// Kernel A.  Rows r >= j.  i = j - p is the number of reflectors already in the panel.
-//  - if i > 0: W[:, i-1] += alpha2 * Vc[:, i-1] with alpha2 = -tau_prev/2 * sum(dot_part)
-//  - a_j[r] -= sum_{k<i} Vc[r,k] W[j,k] + W[r,k] Vc[j,k]
-//  - d[j] = a_j[j]; partial norm over rows > j+1
+// Sum over the 256 threads of a workgroup: xor-shuffles inside each wavefront, then the four
+// wavefront sums in a fixed order.  `s_w` is 4 values of shared memory; two barriers.
 template <typename T>
-__global__ __launch_bounds__(256) void trd_col_update_kernel(T* __restrict__ A, int64_t lda, int n, int p, int j,
-                                                             T* __restrict__ Vc, T* __restrict__ W, int64_t ldw,
-                                                             const T* __restrict__ dot_part, int n_dot_part,
-                                                             const T* __restrict__ tau, T* __restrict__ norm_part,
-                                                             T* __restrict__ d) {
-  constexpr int NB = kTrdNb;
-  __shared__ T red[256];
-  __shared__ T s_wj[NB], s_vj[NB];
-  const int tid = threadIdx.x;
-  const int i = j - p;
-  const int r = j + blockIdx.x * 256 + tid;
-  const bool live = r < n;
-  T alpha2 = T(0);
-  if (i > 0) alpha2 = T(-0.5) * tau[j - 1] * reduce_partials(dot_part, n_dot_part, red);
-  // row j of W and Vc (finalising column i-1 of W on the fly)
-  if (tid < i) {
-    T wv = W[j + (int64_t)tid * ldw];
-    const T vv = Vc[j + (int64_t)tid * ldw];
-    if (tid == i - 1) wv += alpha2 * vv;
-    s_wj[tid] = wv;
-    s_vj[tid] = vv;
-  }
+__device__ __forceinline__ T block_sum_shuffle(T v, T* s_w) {
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m, 64);
+  __syncthreads();  // earlier readers of s_w are done
+  if ((threadIdx.x & 63) == 0) s_w[threadIdx.x >> 6] = v;
   __syncthreads();
-  T x2 = T(0);
-  if (live) {
-    // all 2*NB loads are issued before the first use (fixed trip count, guarded by k < i)
-    T wr[NB], vr[NB];
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {
-      wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
-      vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
-    }
-    T acc = T(0);
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {
-      if (k < i) {
-        T wk = wr[k];
-        if (k == i - 1) {
-          wk += alpha2 * vr[k];
-          // Row j stays unfinished in memory: every workgroup reads it above and adds alpha2
-          // itself, and no later column looks at row j of W again.
-          if (r != j) W[r + (int64_t)k * ldw] = wk;
-        }
-        acc += vr[k] * s_wj[k] + wk * s_vj[k];
-      }
-    }
-    T a = A[r + (int64_t)j * lda];
-    if (i > 0) {
-      a -= acc;
-      A[r + (int64_t)j * lda] = a;
-    }
-    if (r == j) d[j] = a;
-    if (r > j + 1) x2 = a * a;
-  }
-  const T s = block_sum_256(x2, red);
-  if (tid == 0) norm_part[blockIdx.x] = s;
+  return (s_w[0] + s_w[1]) + (s_w[2] + s_w[3]);
 }
 
-// Rows of W below the current column that kernel A of this launch did not touch must also be
-// finalised before the rank-2k update; this runs once per panel after its last column.
+// ---- messages between the workgroups of the fused kernel -------------------------------------
+// A value travels as one (float) or two (double) 64-bit words {32 payload bits, sequence number},
+// each written and read with one single-copy-atomic access: a reader that finds the expected
+// sequence number in a word has that word's payload.
+__device__ __forceinline__ void mail_post(unsigned long long* slot, float value, unsigned seq) {
+  __hip_atomic_store(slot, mailbox_pack(value, seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void mail_post(unsigned long long* slot, double value, unsigned seq) {
+  const unsigned lo = (unsigned)__double2loint(value), hi = (unsigned)__double2hiint(value);
+  __hip_atomic_store(slot, ((unsigned long long)seq << 32) | lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(slot + 1, ((unsigned long long)seq << 32) | hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Polls until the slot carries `seq`; false after kQrSpinLimit polls or once `error` is up.
+template <typename T>
+__device__ __forceinline__ bool mail_fetch(const unsigned long long* slot, unsigned seq, const int* error, T* value) {
+  constexpr bool WIDE = sizeof(T) == 8;
+  unsigned spins = 0;
+  for (;;) {
+    const unsigned long long w0 = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long w1 =
+        WIDE ? __hip_atomic_load(slot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : w0;
+    if ((unsigned)(w0 >> 32) == seq && (unsigned)(w1 >> 32) == seq) {
+      if constexpr (WIDE) *value = __hiloint2double((int)(unsigned)w1, (int)(unsigned)w0);
+      else *value = __uint_as_float((unsigned)w0);
+      return true;
+    }
+    ++spins;
+    if (spins > kQrSpinLimit) return false;
+    if ((spins & 63u) == 0 && __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
+// Sum of the values posted by `nwg` workgroups (thread t fetches workgroup t's) plus one extra
+// value (slot kTrdMaxWg, fetched by thread 255) that comes back in *extra.  All 256 threads call.
+// Returns false if a message did not arrive; `s_fail` and `s_x` are shared scratch.
+template <typename T>
+__device__ __forceinline__ bool mail_gather(const unsigned long long* mail, int nwg, unsigned seq, int* error,
+                                            T* s_w, T* s_x, int* s_fail, T* sum, T* extra) {
+  const int tid = threadIdx.x;
+  T v = T(0);
+  bool ok = true;
+  if (tid < nwg) ok = mail_fetch<T>(mail + 2 * tid, seq, error, &v);
+  if (tid == 255) {
+    T x = T(0);
+    ok = mail_fetch<T>(mail + 2 * kTrdMaxWg, seq, error, &x);
+    *s_x = x;
+  }
+  if (!ok) {
+    __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *s_fail = 1;
+  }
+  *sum = block_sum_shuffle(v, s_w);  // its barriers also publish s_x and s_fail
+  *extra = *s_x;
+  return *s_fail == 0;
+}
+
+// W[r, col] += alpha2 * Vc[r, col] for rows r >= row0: the last w of a panel, which no later
+// column step finishes, before the rank-2k update reads it.
 template <typename T>
 __global__ __launch_bounds__(256) void trd_finish_w_kernel(T* __restrict__ W, const T* __restrict__ Vc, int64_t ldw,
                                                            int n, int row0, int col, const T* __restrict__ dot_part,
@@ -153,66 +165,166 @@ __global__ __launch_bounds__(256) void trd_finish_w_kernel(T* __restrict__ W, co
   W[r + (int64_t)col * ldw] += alpha2 * Vc[r + (int64_t)col * ldw];
 }
 
-// Kernel B.  Rows r >= j+1 (workgroup/thread mapping: r = j + 1 + ...).
+// Steps D(j), A(jn), B(jn) with jn = j + 1, one thread per row r = jn + 256 * workgroup + thread.
+//   do_d    : step D runs (j is a column of this panel whose v and y exist); otherwise the launch
+//             opens a panel at column jn = p and only A and B run
+//   do_next : steps A and B run (jn is still inside the panel); otherwise the launch ends after D
+//             and leaves the unfinished w and the partial sums of w^T v for trd_finish_w_kernel
+// i = j - p is the index of reflector j in the panel; columns k < i of Vc and W are final in memory,
+// column i of W is produced here.  `n_t_part` is the grid size of the launch that ran B(j).
+// `seq` (unique per launch, never 0) tags this launch's messages.
 template <typename T>
-__global__ __launch_bounds__(256) void trd_reflector_kernel(T* __restrict__ A, int64_t lda, int n, int p, int j,
-                                                            T* __restrict__ Vc, T* __restrict__ Vc2,
-                                                            const T* __restrict__ W, int64_t ldw,
-                                                            const T* __restrict__ norm_part, int n_norm_part,
-                                                            T* __restrict__ tau, T* __restrict__ e,
-                                                            T* __restrict__ t_part) {
+__global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int64_t lda, int n, int p, int j,
+                                                         int do_d, int do_next, T* __restrict__ Vc,
+                                                         T* __restrict__ Vc2, T* __restrict__ W, int64_t ldw,
+                                                         const T* __restrict__ y_part, int n_slots,
+                                                         T* __restrict__ t_part, int n_t_part,
+                                                         T* __restrict__ dot_part, T* __restrict__ tau,
+                                                         T* __restrict__ d, T* __restrict__ e,
+                                                         unsigned long long* mail, unsigned seq, int* error) {
   constexpr int NB = kTrdNb;
+  __shared__ T s_t[2 * NB];
+  __shared__ T s_t4[4][2 * NB];
+  __shared__ T s_wj[NB], s_vj[NB];
   __shared__ T s_red[4][2 * NB];
-  __shared__ T red[256];
+  __shared__ T s_w4[4];
+  __shared__ T s_x;
+  __shared__ int s_fail;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int i = j - p;
-  const int r = j + 1 + blockIdx.x * 256 + tid;
+  const int nwg = gridDim.x, wg = blockIdx.x;
+  const int jn = j + 1;
+  const int i = j - p;  // valid when do_d
+  const int r = jn + wg * 256 + tid;
   const bool live = r < n;
-  const T x2 = reduce_partials(norm_part, n_norm_part, red);
-  const T alpha = A[(j + 1) + (int64_t)j * lda];
+  unsigned long long* mail_dot = mail;
+  unsigned long long* mail_norm = mail + 2 * (kTrdMaxWg + 1);
+  if (tid == 0) s_fail = 0;
+
+  T vr[NB], wr[NB];  // this row of Vc and W, columns k < i
+#pragma unroll
+  for (int k = 0; k < NB; ++k) vr[k] = wr[k] = T(0);
+  T vi = T(0), wv = T(0);  // this row of column i: v_j and the unfinished w_j
+  T alpha2 = T(0), w_jn_i = T(0);
+
+  if (do_d) {
+    // ---- D(j): w = tau (y - V (W^T v) - W (V^T v)) ----
+    {
+      // 2*NB columns x n_t_part partials: 4 strided partial sums per column, then 4 adds
+      const int c = tid & (2 * NB - 1), g0 = tid >> 6;
+      T s = T(0);
+      if ((c % NB) < i)
+        for (int g = g0; g < n_t_part; g += 4) s += t_part[(int64_t)g * 2 * NB + c];
+      s_t4[g0][c] = s;
+    }
+    __syncthreads();
+    if (tid < 2 * NB) s_t[tid] = (s_t4[0][tid] + s_t4[1][tid]) + (s_t4[2][tid] + s_t4[3][tid]);
+    __syncthreads();
+    T prod = T(0);
+    if (live) {
+#pragma unroll
+      for (int k = 0; k < NB; ++k) {
+        vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
+        wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
+      }
+      vi = Vc[r + (int64_t)i * ldw];
+      T y = T(0);
+      for (int c0 = 0; c0 < n_slots; c0 += 16) {  // 16 slot loads in flight, summed in slot order
+        T yp[16];
+#pragma unroll
+        for (int c = 0; c < 16; ++c) yp[c] = (c0 + c < n_slots) ? y_part[(int64_t)(c0 + c) * n + r] : T(0);
+#pragma unroll
+        for (int c = 0; c < 16; ++c) y += yp[c];
+      }
+      T corr = T(0);
+#pragma unroll
+      for (int k = 0; k < NB; ++k) corr += vr[k] * s_t[k] + wr[k] * s_t[NB + k];
+      wv = tau[j] * (y - corr);
+      prod = wv * vi;
+    }
+    const T dot = block_sum_shuffle(prod, s_w4);
+    if (!do_next) {
+      if (live) W[r + (int64_t)i * ldw] = wv;
+      if (tid == 0) dot_part[wg] = dot;
+      return;
+    }
+    if (tid == 0) mail_post(mail_dot + 2 * wg, dot, seq);
+    if (r == jn) mail_post(mail_dot + 2 * kTrdMaxWg, wv, seq);  // the unfinished W[jn, i]
+    T total, w_jn_raw;
+    if (!mail_gather<T>(mail_dot, nwg, seq, error, s_w4, &s_x, &s_fail, &total, &w_jn_raw)) return;
+    alpha2 = T(-0.5) * tau[j] * total;
+    w_jn_i = w_jn_raw + alpha2;  // v_j has its unit entry in row jn
+  }
+
+  // ---- A(jn): finish w_j, bring column jn up to date, norm of its sub-column ----
+  const int in = jn - p;  // reflectors in the panel before column jn
+  T wf = T(0);
+  if (do_d) {
+    wf = wv + alpha2 * vi;
+    if (live) W[r + (int64_t)i * ldw] = wf;
+    if (tid < i) {  // row jn of the finished columns
+      s_wj[tid] = W[jn + (int64_t)tid * ldw];
+      s_vj[tid] = Vc[jn + (int64_t)tid * ldw];
+    }
+    __syncthreads();
+  }
+  T a = T(0), x2 = T(0);
+  if (live) {
+    a = A[r + (int64_t)jn * lda];
+    if (do_d) {
+      T acc = vi * w_jn_i + wf;  // column i: Vc[r,i] W[jn,i] + W[r,i] Vc[jn,i], Vc[jn,i] = 1
+#pragma unroll
+      for (int k = 0; k < NB; ++k)
+        if (k < i) acc += vr[k] * s_wj[k] + wr[k] * s_vj[k];
+      a -= acc;
+      A[r + (int64_t)jn * lda] = a;
+    }
+    if (r == jn) d[jn] = a;
+    if (r > jn + 1) x2 = a * a;
+  }
+  if (jn >= n - 1) return;  // the last column has no reflector
+  const T norm_part = block_sum_shuffle(x2, s_w4);
+  if (tid == 0) mail_post(mail_norm + 2 * wg, norm_part, seq);
+  if (r == jn + 1) mail_post(mail_norm + 2 * kTrdMaxWg, a, seq);  // alpha
+  T x2_total, alpha;
+  if (!mail_gather<T>(mail_norm, nwg, seq, error, s_w4, &s_x, &s_fail, &x2_total, &alpha)) return;
+
+  // ---- B(jn): reflector, v, partial W^T v and V^T v ----
   T beta = alpha, tauv = T(0), scale = T(0);
-  if (x2 > T(0)) {
-    const T nrm = sqrt(alpha * alpha + x2);
+  if (x2_total > T(0)) {
+    const T nrm = sqrt(alpha * alpha + x2_total);
     beta = (alpha >= T(0)) ? -nrm : nrm;
     tauv = (beta - alpha) / beta;
     scale = T(1) / (alpha - beta);
   }
   T v = T(0);
-  if (live) {
-    if (r == j + 1) {
+  if (live && r > jn) {
+    if (r == jn + 1) {
       v = T(1);
+      tau[jn] = tauv;
+      e[jn] = beta;
     } else {
-      v = A[r + (int64_t)j * lda] * scale;
+      v = a * scale;
+      A[r + (int64_t)jn * lda] = v;  // reflector kept for the back-transformation
     }
   }
-  // everything that reads A[j+1, j] has done so before it is overwritten below
-  __syncthreads();
-  if (live) {
-    if (r == j + 1) {
-      tau[j] = tauv;
-      e[j] = beta;
-    } else {
-      A[r + (int64_t)j * lda] = v;  // reflector kept for the back-transformation
-    }
-    Vc[r + (int64_t)i * ldw] = v;
-    Vc2[r + (int64_t)i * ldw] = v;
+  if (live) {  // row jn reads as zero, like the rows above it
+    Vc[r + (int64_t)in * ldw] = v;
+    Vc2[r + (int64_t)in * ldw] = v;
   }
-  // rows <= j of this column of Vc must read as zero for later row-j lookups
-  if (blockIdx.x == 0) {
-    for (int rr = p + tid; rr <= j; rr += 256) {
-      Vc[rr + (int64_t)i * ldw] = T(0);
-      Vc2[rr + (int64_t)i * ldw] = T(0);
+  if (wg == 0) {
+    for (int rr = p + tid; rr < jn; rr += 256) {
+      Vc[rr + (int64_t)in * ldw] = T(0);
+      Vc2[rr + (int64_t)in * ldw] = T(0);
     }
   }
-  // partial W^T v and V^T v over this workgroup's rows (columns k < i): 2*NB products per thread,
-  // two 32-value butterflies per wavefront
   {
     T pw[NB], pv[NB];
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
-      const bool on = live && k < i;
-      pw[k] = on ? W[r + (int64_t)k * ldw] * v : T(0);
-      pv[k] = on ? Vc[r + (int64_t)k * ldw] * v : T(0);
+      const T wk = (do_d && k == i) ? wf : wr[k];  // wr, vr are zero beyond column i
+      const T vk = (do_d && k == i) ? vi : vr[k];
+      pw[k] = wk * v;
+      pv[k] = vk * v;
     }
     const T tw = wave_reduce_32<T>(pw, lane);
     const T tv = wave_reduce_32<T>(pv, lane);
@@ -222,12 +334,17 @@ __global__ __launch_bounds__(256) void trd_reflector_kernel(T* __restrict__ A, i
     }
   }
   __syncthreads();
-  if (tid < 2 * NB) {
-    const int k = tid % NB;
-    T s = T(0);
-    if (k < i) s = s_red[0][tid] + s_red[1][tid] + s_red[2][tid] + s_red[3][tid];
-    t_part[(int64_t)blockIdx.x * 2 * NB + tid] = s;
-  }
+  if (tid < 2 * NB)
+    t_part[(int64_t)wg * 2 * NB + tid] = (s_red[0][tid] + s_red[1][tid]) + (s_red[2][tid] + s_red[3][tid]);
+}
+
+// d[0..n) <- NaN if a workgroup of trd_column_kernel gave up waiting: the eigenvalues then come
+// out as NaN instead of silently wrong.
+template <typename T>
+__global__ void trd_poison_on_error_kernel(T* __restrict__ d, int n, const int* __restrict__ error) {
+  if (*error == 0) return;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) d[i] = T(NAN);
 }
 
 // Kernel C.  The trailing matrix (rows and columns o = j+1 .. n-1, only its lower triangle is
@@ -302,58 +419,6 @@ __global__ __launch_bounds__(256) void trd_symv_kernel(const T* __restrict__ A, 
   }
 }
 
-// Kernel D.  Rows r >= j+1.
-template <typename T>
-__global__ __launch_bounds__(256) void trd_w_kernel(int n, int p, int j, const T* __restrict__ Vc, T* __restrict__ W,
-                                                    int64_t ldw, const T* __restrict__ y_part, int n_chunks,
-                                                    const T* __restrict__ t_part, int n_t_part,
-                                                    const T* __restrict__ tau, T* __restrict__ dot_part) {
-  constexpr int NB = kTrdNb;
-  __shared__ T red[256];
-  __shared__ T s_t[2 * NB];
-  __shared__ T s_t4[4][2 * NB];
-  const int tid = threadIdx.x;
-  const int i = j - p;
-  const int r = j + 1 + blockIdx.x * 256 + tid;
-  {
-    // 2*NB columns x n_t_part partials: 4 strided partial sums per column, then 4 adds
-    const int c = tid & (2 * NB - 1), g0 = tid >> 6;
-    T s = T(0);
-    if ((c % NB) < i)
-      for (int g = g0; g < n_t_part; g += 4) s += t_part[(int64_t)g * 2 * NB + c];
-    s_t4[g0][c] = s;
-  }
-  __syncthreads();
-  if (tid < 2 * NB) s_t[tid] = (s_t4[0][tid] + s_t4[1][tid]) + (s_t4[2][tid] + s_t4[3][tid]);
-  __syncthreads();
-  T prod = T(0);
-  if (r < n) {
-    T wr[NB], vr[NB];
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {
-      vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
-      wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
-    }
-    T y = T(0);
-    for (int c0 = 0; c0 < n_chunks; c0 += 16) {  // 16 slot loads in flight, summed in slot order
-      T yp[16];
-#pragma unroll
-      for (int c = 0; c < 16; ++c) yp[c] = (c0 + c < n_chunks) ? y_part[(int64_t)(c0 + c) * n + r] : T(0);
-#pragma unroll
-      for (int c = 0; c < 16; ++c) y += yp[c];
-    }
-    T corr = T(0);
-#pragma unroll
-    for (int k = 0; k < NB; ++k) corr += vr[k] * s_t[k] + wr[k] * s_t[NB + k];
-    const T wv = tau[j] * (y - corr);
-    W[r + (int64_t)i * ldw] = wv;
-    prod = wv * Vc[r + (int64_t)i * ldw];
-  }
-  const T s = block_sum_256(prod, red);
-  if (tid == 0) dot_part[blockIdx.x] = s;
-}
-
-// d[n-1] after all updates: the last column has no reflector of its own.
 // Tridiagonalise A (n x n, lower triangle referenced; destroyed).  On exit d[0..n), e[0..n-1),
 // tau[0..n-1) and, below the first subdiagonal of A, the reflector vectors (implicit unit at
 // row j+1 of column j), as LAPACK sytrd('L') leaves them.
@@ -365,37 +430,45 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
     SOAPMI_HIP(hipMemcpyAsync(d, A, sizeof(T), hipMemcpyDeviceToDevice, s));
     return kOk;
   }
-  int last_dot_parts = 0;  // number of dot partials produced by the latest kernel D
+  SOAPMI_REQUIRE(ceil_div64(n, 256) <= kTrdMaxWg, "matrix size %d exceeds what the column kernel supports", n);
+  {
+    // messages of an earlier factorisation in the same workspace must not be mistaken for new ones
+    const int words = 2 * (2 * (kTrdMaxWg + 1) * 2 + 2);
+    hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3((words + 255) / 256), dim3(256), 0, s,
+                       reinterpret_cast<unsigned*>(ws.mail), words);
+  }
+  unsigned seq = 0;
   for (int p = 0; p < n; p += NB) {
     const int pe = std::min(n, p + NB);
-    int cols_done = 0;
+    // open the panel: A(p), B(p)
+    int grid = (int)ceil_div64(n - p, 256);
+    hipLaunchKernelGGL((trd_column_kernel<T>), dim3(grid), dim3(256), 0, s, A, lda, n, p, p - 1, 0, 1, ws.vc, ws.vc2,
+                       ws.w, ldw, ws.y_part, 0, ws.t_part, 0, ws.dot_part, tau, d, e, ws.mail, ++seq, ws.error);
+    int t_parts = grid;  // grid of the launch that ran B for the current column
+    int cols_done = 0, last_dot_parts = 0;
     for (int j = p; j < pe; ++j) {
+      if (j == n - 1) break;  // only the diagonal entry remained, and A(n-1) has stored it
       const int i = j - p;
-      const int nwgA = (int)ceil_div64(n - j, 256);
-      hipLaunchKernelGGL((trd_col_update_kernel<T>), dim3(nwgA), dim3(256), 0, s, A, lda, n, p, j, ws.vc, ws.w, ldw,
-                         ws.dot_part, last_dot_parts, tau, ws.norm_part, d);
-      if (j == n - 1) break;  // only the diagonal entry remained
       const int nt = n - j - 1;
-      const int nwgB = (int)ceil_div64(nt, 256);
-      hipLaunchKernelGGL((trd_reflector_kernel<T>), dim3(nwgB), dim3(256), 0, s, A, lda, n, p, j, ws.vc, ws.vc2, ws.w,
-                         ldw, ws.norm_part, nwgA, tau, e, ws.t_part);
       const int nb = (int)ceil_div64(nt, kTrdTile);
       hipLaunchKernelGGL((trd_symv_kernel<T>), dim3(nb * (nb + 1) / 2), dim3(256), 0, s, A, lda, n, j,
                          ws.vc + (int64_t)i * ldw, ws.y_part);
-      hipLaunchKernelGGL((trd_w_kernel<T>), dim3(nwgB), dim3(256), 0, s, n, p, j, ws.vc, ws.w, ldw, ws.y_part, nb,
-                         ws.t_part, nwgB, tau, ws.dot_part);
-      last_dot_parts = nwgB;
+      grid = (int)ceil_div64(nt, 256);
+      const int do_next = (j + 1 < pe) ? 1 : 0;
+      hipLaunchKernelGGL((trd_column_kernel<T>), dim3(grid), dim3(256), 0, s, A, lda, n, p, j, 1, do_next, ws.vc, ws.vc2,
+                         ws.w, ldw, ws.y_part, nb, ws.t_part, t_parts, ws.dot_part, tau, d, e, ws.mail, ++seq,
+                         ws.error);
+      t_parts = grid;
+      last_dot_parts = grid;
       cols_done = i + 1;
     }
     SOAPMI_LAUNCH_CHECK();
     if (pe >= n) break;
-    // finish the last w of the panel, then A[pe:, pe:] -= V W^T + W V^T on the full square
+    // finish the last w of the panel, then A[pe:, pe:] -= [V | W] [W | V]^T on the lower tiles
     const int jl = pe - 1;
     hipLaunchKernelGGL((trd_finish_w_kernel<T>), dim3((unsigned)ceil_div64(n - pe, 256)), dim3(256), 0, s, ws.w, ws.vc,
                        ldw, n, pe, cols_done - 1, ws.dot_part, last_dot_parts, tau + jl);
-    last_dot_parts = 0;
     const int nt = n - pe;
-    // A[pe:, pe:] -= [V | W] [W | V]^T, tiles on or below the diagonal only
     int rc;
     if (cols_done == NB) {
       rc = gemm_lower<T>(s, 0, 1, nt, 2 * NB, T(-1), ws.vc + pe, ldw, ws.w + pe, ldw, T(1), A + pe + (int64_t)pe * lda,
@@ -410,6 +483,9 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
       if (rc) return rc;
     }
   }
+  hipLaunchKernelGGL((trd_poison_on_error_kernel<T>), dim3((unsigned)ceil_div64(n, 256)), dim3(256), 0, s, d, n,
+                     ws.error);
+  SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
 
