@@ -33,6 +33,8 @@ struct DcWorkspace {
   T* wv;     // n   matching z components
   T* dnew;   // n
   T* zhat;   // n
+  T* mu;     // n   root offsets from their origin poles (wavefront-per-root path)
+  int* org;  // n   origin pole of each root
   T* rot_c;  // n
   T* rot_s;  // n
   T* skey;   // 4n  sort keys
@@ -59,6 +61,8 @@ static inline void dc_workspace_layout(WS& ws, int64_t n, DcWorkspace<T>* out) {
   w.wv = ws.template take<T>(n);
   w.dnew = ws.template take<T>(n);
   w.zhat = ws.template take<T>(n);
+  w.mu = ws.template take<T>(n);
+  w.org = ws.template take<int>(n);
   w.rot_c = ws.template take<T>(n);
   w.rot_s = ws.template take<T>(n);
   w.skey = ws.template take<T>(4 * n + 8);
@@ -405,6 +409,129 @@ __device__ void dc_secular_root(int i, int k, const T* __restrict__ dl, const T*
   for (int j = 0; j < k; ++j) delta[(int64_t)j * dstride] = (dl[j] - dorg) - mu;
 }
 
+// The same iteration with the sums over the poles spread over the 64 lanes of a wavefront (lane l
+// takes poles l, l + 64, ...; xor-butterfly sums give every lane the same total), for merges with
+// many poles, where a thread per root leaves most of the chip idle.  Writes the root, its origin
+// pole and its offset; dc_delta_kernel then forms the differences with lanes along the roots.
+template <typename T>
+__device__ __forceinline__ T dc_wave_sum(T v) {
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m, 64);
+  return v;
+}
+
+template <typename T>
+__device__ void dc_secular_root_wave(int i, int k, int lane, const T* __restrict__ dl, const T* __restrict__ w, T rho,
+                                     T* lam_out, T* mu_out, int* org_out) {
+  const T eps = std::numeric_limits<T>::epsilon();
+  if (k == 1) {
+    const T mu = rho * w[0] * w[0];
+    if (lane == 0) { *lam_out = dl[0] + mu; *mu_out = mu; *org_out = 0; }
+    return;
+  }
+  const T di = dl[i];
+  int org, p1, p2, split;
+  T lo, hi;
+  if (i < k - 1) {
+    const T gap = dl[i + 1] - di;
+    const T half = T(0.5) * gap;
+    T f = T(0);
+    for (int j = lane; j < k; j += 64) f += rho * w[j] * w[j] / ((dl[j] - di) - half);
+    f = T(1) + dc_wave_sum(f);
+    if (f >= T(0)) { org = i; lo = T(0); hi = half; }
+    else { org = i + 1; lo = -half; hi = T(0); }
+    p1 = i; p2 = i + 1; split = i;
+  } else {
+    T s = T(0);
+    for (int j = lane; j < k; j += 64) s += w[j] * w[j];
+    s = dc_wave_sum(s);
+    org = k - 1; lo = T(0); hi = rho * s;
+    p1 = k - 2; p2 = k - 1; split = k - 2;
+  }
+  const T dorg = dl[org];
+  T mu = T(0.5) * (lo + hi);
+  for (int it = 0; it < 120; ++it) {
+    if (!(mu > lo && mu < hi)) break;
+    T psi = T(0), phi = T(0), dpsi = T(0), dphi = T(0), err = T(0);
+    for (int j = lane; j < k; j += 64) {
+      const T den = (dl[j] - dorg) - mu;
+      const T tj = rho * w[j] * w[j] / den;
+      const T tt = tj / den;
+      if (j <= split) { psi += tj; dpsi += tt; }
+      else { phi += tj; dphi += tt; }
+      err += fabs(tj);
+    }
+    psi = dc_wave_sum(psi); phi = dc_wave_sum(phi); dpsi = dc_wave_sum(dpsi); dphi = dc_wave_sum(dphi);
+    err = T(1) + dc_wave_sum(err);
+    const T g = T(1) + psi + phi;
+    if (fabs(g) <= T(16) * eps * err) break;
+    if (g > T(0)) hi = mu; else lo = mu;
+    if (hi - lo <= T(2) * eps * fmax(fabs(lo), fabs(hi))) break;
+    const T D1 = (dl[p1] - dorg) - mu, D2 = (dl[p2] - dorg) - mu;
+    const T C = g - D1 * dpsi - D2 * dphi;
+    const T A = (D1 + D2) * g - D1 * D2 * (dpsi + dphi);
+    const T B = D1 * D2 * g;
+    T best = mu;
+    bool found = false;
+    T cand[2];
+    int nc = 0;
+    if (C == T(0)) {
+      if (A != T(0)) cand[nc++] = B / A;
+    } else {
+      const T disc = A * A - T(4) * B * C;
+      if (disc >= T(0)) {
+        const T sq = sqrt(disc);
+        const T qq = (A >= T(0)) ? A + sq : A - sq;
+        cand[nc++] = qq / (T(2) * C);
+        if (qq != T(0)) cand[nc++] = T(2) * B / qq;
+      }
+    }
+    for (int c = 0; c < nc; ++c) {
+      const T x = mu + cand[c];
+      if (x > lo && x < hi && (!found || fabs(cand[c]) < fabs(best - mu))) { best = x; found = true; }
+    }
+    if (!found) {
+      if (lo > T(0) && hi > T(16) * lo) best = sqrt(lo) * sqrt(hi);
+      else if (hi < T(0) && lo < T(16) * hi) best = -(sqrt(-lo) * sqrt(-hi));
+      else best = T(0.5) * (lo + hi);
+      if (!(best > lo && best < hi)) break;
+    }
+    mu = best;
+  }
+  if (!(mu > lo && mu < hi)) mu = T(0.5) * (lo + hi);
+  if (lane == 0) { *lam_out = dorg + mu; *mu_out = mu; *org_out = org; }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dc_secular_wave_kernel(int t, int n, const T* __restrict__ e,
+                                                              const T* __restrict__ dl, const T* __restrict__ wv,
+                                                              const int* __restrict__ kcount, T* __restrict__ dnew,
+                                                              T* __restrict__ mu, int* __restrict__ org) {
+  const int q = blockIdx.y;
+  const int k = kcount[q];
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);  // one wavefront per root
+  if (i >= k) return;
+  const DcMerge m = dc_merge(t, q, n);
+  const T rho = T(2) * fabs(e[m.mid - 1]);
+  dc_secular_root_wave<T>(i, k, threadIdx.x & 63, dl + m.lo, wv + m.lo, rho, dnew + m.lo + i, mu + m.lo + i,
+                          org + m.lo + i);
+}
+
+// deltaT[i, j] = (dl_j - dl_org(i)) - mu_i at S[(lo + i) + (lo + j) * lds]: lanes along the roots.
+template <typename T>
+__global__ __launch_bounds__(256) void dc_delta_kernel(int t, int n, const T* __restrict__ dl,
+                                                       const int* __restrict__ kcount, const T* __restrict__ mu,
+                                                       const int* __restrict__ org, T* __restrict__ S, int64_t lds) {
+  const int q = blockIdx.z;
+  const int k = kcount[q];
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= k) return;
+  const int lo = dc_bound(t, q, n);
+  const T dorg = dl[lo + org[lo + i]], m = mu[lo + i];
+  T* row = S + (lo + i) + (int64_t)lo * lds;
+  for (int j = blockIdx.y; j < k; j += gridDim.y) row[(int64_t)j * lds] = (dl[lo + j] - dorg) - m;
+}
+
 template <typename T>
 __global__ __launch_bounds__(64) void dc_secular_kernel(int t, int n, const T* __restrict__ e,
                                                         const T* __restrict__ dl, const T* __restrict__ wv,
@@ -573,8 +700,15 @@ static inline int stedc(hipStream_t s, int n, const T* d0, const T* e0, T* w_out
                        ws.rot_c, ws.rot_s, ws.nrot);
     hipLaunchKernelGGL((dc_gather_kernel<T>), dim3(rbl, ycols, nq), dim3(256), 0, s, t, n, ws.X, ws.ldx, Y, ldy, ws.idx,
                        ws.kcount);
-    hipLaunchKernelGGL((dc_secular_kernel<T>), dim3((unsigned)ceil_div64(nmax, 64), nq), dim3(64), 0, s, t, n, ws.e,
-                       ws.dl, ws.wv, ws.kcount, ws.dnew, ws.S, ws.lds);
+    if (nmax >= 256) {
+      hipLaunchKernelGGL((dc_secular_wave_kernel<T>), dim3((unsigned)ceil_div64(nmax, 4), nq), dim3(256), 0, s, t, n,
+                         ws.e, ws.dl, ws.wv, ws.kcount, ws.dnew, ws.mu, ws.org);
+      hipLaunchKernelGGL((dc_delta_kernel<T>), dim3(rbl, ycols, nq), dim3(256), 0, s, t, n, ws.dl, ws.kcount, ws.mu,
+                         ws.org, ws.S, ws.lds);
+    } else {
+      hipLaunchKernelGGL((dc_secular_kernel<T>), dim3((unsigned)ceil_div64(nmax, 64), nq), dim3(64), 0, s, t, n, ws.e,
+                         ws.dl, ws.wv, ws.kcount, ws.dnew, ws.S, ws.lds);
+    }
     hipLaunchKernelGGL((dc_zhat_kernel<T>), dim3(nmax, nq), dim3(256), 0, s, t, n, ws.dl, ws.wv, ws.kcount, ws.S, ws.lds,
                        ws.zhat);
     hipLaunchKernelGGL((dc_form_u_kernel<T>), dim3(rbl, nq), dim3(256), 0, s, t, n, ws.kcount, ws.zhat, ws.S, ws.lds);
