@@ -45,6 +45,12 @@ void soapmi_world_rank_and_size(int* rank, int* size);
 
 const char* soapmi_last_error(void);
 
+/* Process-wide tuning knobs (no counterpart in the reference).  Options:
+ *   "qr_persistent_max_workgroups"  0..128 (default 128): a QR panel whose grid (rows / 256) fits
+ *       runs as one persistent launch whose workgroups exchange partial sums through device memory;
+ *       larger panels, or all panels with 0, run one launch per column instead. */
+int soapmi_set_option(const char* name, int64_t value);
+
 /* ---- Gram preconditioner EMA ---------------------------------------------------------- */
 
 /* P <- lerp(P, G G^T, 1-beta) (side 0, P is rows x rows) or lerp(P, G^T G, 1-beta) (side 1,

@@ -1,6 +1,7 @@
 // extern "C" surface of libsoap_mi355.so (declared in include/soap_mi355.h).
 #include <stdarg.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "../../include/soap_mi355.h"
@@ -29,6 +30,8 @@ struct InternalScratch {
   size_t size = 0;
 };
 static InternalScratch g_scratch[64];
+// largest grid for which the QR panel runs as one persistent launch (see soapmi_set_option)
+static std::atomic<int> g_qr_persistent_max_wg{kQrPersistentMaxWg};
 static std::mutex g_scratch_mutex;
 
 static int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out) {
@@ -142,6 +145,18 @@ void soapmi_world_rank_and_size(int* rank, int* size) {
 }
 
 const char* soapmi_last_error(void) { return last_error(); }
+
+int soapmi_set_option(const char* name, int64_t value) {
+  SOAPMI_REQUIRE(name, "option name must not be null");
+  if (strcmp(name, "qr_persistent_max_workgroups") == 0) {
+    SOAPMI_REQUIRE(value >= 0 && value <= kQrPersistentMaxWg, "qr_persistent_max_workgroups must be in 0..%d",
+                   kQrPersistentMaxWg);
+    g_qr_persistent_max_wg.store((int)value);
+    return kOk;
+  }
+  set_error("unknown option '%s'", name);
+  return kInvalidArgument;
+}
 
 int soapmi_gemm_f32(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const float* a,
                     int64_t lda, const float* b, int64_t ldb, float beta, float* c, int64_t ldc, void* stream) {
@@ -470,7 +485,8 @@ int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t 
   Workspace w(ws, need);
   QrWorkspace<float> qws;
   qr_workspace_layout<float>(w, n, &qws);
-  return qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws);
+  return qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws,
+                                     g_qr_persistent_max_wg.load());
 }
 
 size_t soapmi_power_iteration_qr_workspace_bytes(int64_t n) {

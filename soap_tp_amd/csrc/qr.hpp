@@ -612,7 +612,7 @@ static inline size_t qr_workspace_bytes(int64_t n) {
 // whose products have K = 128 and run on the full-size MFMA tile.
 template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
-                                       const QrWorkspace<T>& ws) {
+                                       const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg) {
   const int NB = kQrNb, OB = kBrMax;
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
@@ -638,7 +638,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       const int nwg = (int)ceil_div64(rows, 256);
       T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
       T* piv[2] = {ws.piv, ws.piv + NB};
-      if (nwg <= kQrPersistentMaxWg) {
+      if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
                            ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg);
         seq_base += (unsigned)nbw;

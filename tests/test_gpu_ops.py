@@ -153,6 +153,29 @@ def test_estimated_order_qr_and_power_iteration(size, device):
     torch.testing.assert_close(q_dev.T @ q_dev, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("size", [40, 300, 700])
+def test_qr_launch_per_column_panel_path(size, device):
+    """The panel factorisation used beyond 128 workgroups (n > 32768), forced at small sizes."""
+    from soap_tp_amd import _native
+    matrix = make_matrix(size, size, seed=SEED + 31 * size)
+    results = []
+    try:
+        for limit in (0, 128):
+            _native.call("soapmi_set_option", b"qr_persistent_max_workgroups", limit)
+            factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+            ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
+            results.append(factor.cpu())
+    finally:
+        _native.call("soapmi_set_option", b"qr_persistent_max_workgroups", 128)
+    expected_q = oracle.householder_qr(matrix)
+    for factor in results:
+        assert relative_l2(factor, expected_q) <= 5e-5
+        torch.testing.assert_close(factor.T @ factor, torch.eye(size), rtol=1e-4, atol=1e-4)
+    assert relative_l2(results[0], results[1]) <= 1e-5
+    with pytest.raises(ValueError):
+        _native.call("soapmi_set_option", b"qr_persistent_max_workgroups", 129)
+
+
 def test_argsort_ties_and_large(device):
     from soap_tp_amd import _native
     for count in (1, 2, 33, 4096, 16384, 20000):
