@@ -48,7 +48,11 @@ const char* soapmi_last_error(void);
 /* Process-wide tuning knobs (no counterpart in the reference).  Options:
  *   "qr_persistent_max_workgroups"  0..128 (default 128): a QR panel whose grid (rows / 256) fits
  *       runs as one persistent launch whose workgroups exchange partial sums through device memory;
- *       larger panels, or all panels with 0, run one launch per column instead. */
+ *       larger panels, or all panels with 0, run one launch per column instead.
+ *   "message_spin_limit"  0..4194304 (default 4194304): how many times a workgroup of the QR panel
+ *       kernel or of the tridiagonalisation's column kernel polls for another workgroup's message
+ *       before it gives up.  Giving up never hangs and never passes silently: the kernels leave,
+ *       and the factorisation's output is poisoned with NaN (Q's diagonal, the eigenvalues). */
 int soapmi_set_option(const char* name, int64_t value);
 
 /* ---- Gram preconditioner EMA ---------------------------------------------------------- */

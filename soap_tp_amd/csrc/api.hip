@@ -32,6 +32,8 @@ struct InternalScratch {
 static InternalScratch g_scratch[64];
 // largest grid for which the QR panel runs as one persistent launch (see soapmi_set_option)
 static std::atomic<int> g_qr_persistent_max_wg{kQrPersistentMaxWg};
+// polls a workgroup spends waiting for another one's message before it gives up (see soapmi_set_option)
+static std::atomic<unsigned> g_message_spin_limit{kQrSpinLimit};
 static std::mutex g_scratch_mutex;
 
 static int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out) {
@@ -132,7 +134,8 @@ static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_
   Workspace w(ws, need);
   EighWorkspace<T> ews;
   eigh_workspace_layout<T>(w, n, &ews);
-  return eigh_ascending<T>((hipStream_t)stream, a, lda, eigenvalues, q, ldq, (int)n, ews);
+  return eigh_ascending<T>((hipStream_t)stream, a, lda, eigenvalues, q, ldq, (int)n, ews,
+                           g_message_spin_limit.load());
 }
 
 extern "C" {
@@ -152,6 +155,11 @@ int soapmi_set_option(const char* name, int64_t value) {
     SOAPMI_REQUIRE(value >= 0 && value <= kQrPersistentMaxWg, "qr_persistent_max_workgroups must be in 0..%d",
                    kQrPersistentMaxWg);
     g_qr_persistent_max_wg.store((int)value);
+    return kOk;
+  }
+  if (strcmp(name, "message_spin_limit") == 0) {
+    SOAPMI_REQUIRE(value >= 0 && value <= (int64_t)kQrSpinLimit, "message_spin_limit must be in 0..%u", kQrSpinLimit);
+    g_message_spin_limit.store((unsigned)value);
     return kOk;
   }
   set_error("unknown option '%s'", name);
@@ -486,7 +494,7 @@ int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t 
   QrWorkspace<float> qws;
   qr_workspace_layout<float>(w, n, &qws);
   return qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws,
-                                     g_qr_persistent_max_wg.load());
+                                     g_qr_persistent_max_wg.load(), g_message_spin_limit.load());
 }
 
 size_t soapmi_power_iteration_qr_workspace_bytes(int64_t n) {

@@ -43,18 +43,31 @@ static inline size_t eigh_workspace_bytes(int64_t n) {
   return sizer.total();
 }
 
+// w[0..n) and the diagonal of Z <- NaN if the tridiagonalisation reported lost messages: the
+// decomposition is then unusable, and this makes it impossible to miss.
+template <typename T>
+__global__ void eigh_poison_on_error_kernel(T* __restrict__ w, T* __restrict__ Z, int64_t ldz, int n,
+                                            const int* __restrict__ error) {
+  if (*error == 0) return;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    w[i] = T(NAN);
+    Z[i + (int64_t)i * ldz] = T(NAN);
+  }
+}
+
 // A (n x n, lower triangle referenced, destroyed) = Z diag(w) Z^T, w ascending.
 template <typename T>
 static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, int64_t ldz, int n,
-                                 const EighWorkspace<T>& ws) {
+                                 const EighWorkspace<T>& ws, unsigned spin_limit = kQrSpinLimit) {
   if (n <= 0) return kOk;
-  int rc = sytrd_lower<T>(s, A, lda, n, ws.d, ws.e, ws.tau, ws.trd);
+  int rc = sytrd_lower<T>(s, A, lda, n, ws.d, ws.e, ws.tau, ws.trd, spin_limit);
   if (rc) return rc;
   rc = stedc<T>(s, n, ws.d, ws.e, w, Z, ldz, ws.dc);
   if (rc) return rc;
   // Z <- H_0 H_1 ... H_{n-2} Z, 128-wide block reflectors applied last block first.
   const int nref = n - 1;  // reflector j lives in column j, rows j+1..n-1
-  if (nref <= 0) return kOk;
+  if (nref <= 0) return kOk;  // n == 1: no column kernel ran
   constexpr int OB = kBrMax;
   const int blocks = (int)ceil_div64(nref, OB);
   const int64_t ldv = n;
@@ -68,6 +81,9 @@ static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, i
     rc = apply_block_reflector<T>(s, ws.br, ws.t_block, false, rows, nbw, n, ldv, Z + (p + 1), ldz);
     if (rc) return rc;
   }
+  hipLaunchKernelGGL((eigh_poison_on_error_kernel<T>), dim3((unsigned)ceil_div64(n, 256)), dim3(256), 0, s, w, Z, ldz, n,
+                     ws.trd.error);
+  SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
 

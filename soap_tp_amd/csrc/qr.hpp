@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
 // workgroup's column c+1, which those wrote after they had read column c.
 // Requirements: all workgroups of the launch are resident at the same time (the host launches at
 // most kQrPersistentMaxWg of them, one per CU).  Waiting is bounded: a thread that does not see a
-// word arrive within kQrSpinLimit polls raises `error`, and every workgroup that sees the flag or
+// word arrive within `spin_limit` polls (kQrSpinLimit unless the caller lowers it) raises `error`, and every workgroup that sees the flag or
 // runs out of patience itself leaves the kernel.
 constexpr int kQrPersistentMaxWg = 128;
 constexpr unsigned kQrSpinLimit = 1u << 22;
@@ -215,7 +215,8 @@ __device__ __forceinline__ unsigned long long mailbox_pack(float value, unsigned
 // error flag is up.
 template <int COUNT>
 __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&slot)[COUNT], const bool (&used)[COUNT],
-                                             unsigned seq, const int* error, float (&value)[COUNT]) {
+                                             unsigned seq, const int* error, unsigned spin_limit,
+                                             float (&value)[COUNT]) {
   unsigned spins = 0;
   for (;;) {
     unsigned long long word[COUNT];
@@ -232,7 +233,7 @@ __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&s
       return true;
     }
     ++spins;
-    if (spins > kQrSpinLimit) return false;
+    if (spins > spin_limit) return false;
     if ((spins & 63u) == 0 && __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
     __builtin_amdgcn_s_sleep(1);
   }
@@ -241,7 +242,8 @@ __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&s
 __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restrict__ A, int64_t lda, int n, int p,
                                                                   int pe, unsigned long long* part,
                                                                   unsigned long long* piv, float* __restrict__ tau,
-                                                                  unsigned seq_base, int* error, int nwg) {
+                                                                  unsigned seq_base, int* error, int nwg,
+                                                                  unsigned spin_limit) {
   using T = float;
   constexpr int NB = kQrNb;
   __shared__ T s_tc[NB];
@@ -302,7 +304,7 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
           used[u] = w0 + 8 * u < nwg;
           slot[u] = part_c + (used[u] ? (w0 + 8 * u) : 0) * NB + k;
         }
-        ok = mailbox_wait<8>(slot, used, seq, error, v);
+        ok = mailbox_wait<8>(slot, used, seq, error, spin_limit, v);
 #pragma unroll
         for (int u = 0; u < 8; ++u) s += v[u];
       }
@@ -311,7 +313,7 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
         const unsigned long long* slot[1] = {piv_c + tid};
         const bool used[1] = {true};
         float v[1];
-        ok = mailbox_wait<1>(slot, used, seq, error, v);
+        ok = mailbox_wait<1>(slot, used, seq, error, spin_limit, v);
         s_piv[tid] = v[0];
       }
       if (!ok) {
@@ -612,7 +614,8 @@ static inline size_t qr_workspace_bytes(int64_t n) {
 // whose products have K = 128 and run on the full-size MFMA tile.
 template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
-                                       const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg) {
+                                       const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
+                                       unsigned spin_limit = kQrSpinLimit) {
   const int NB = kQrNb, OB = kBrMax;
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
@@ -640,7 +643,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       T* piv[2] = {ws.piv, ws.piv + NB};
       if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
-                           ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg);
+                           ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit);
         seq_base += (unsigned)nbw;
       } else {
         for (int j = p - 1; j < pe; ++j) {

@@ -107,9 +107,10 @@ __device__ __forceinline__ void mail_post(unsigned long long* slot, double value
   __hip_atomic_store(slot + 1, ((unsigned long long)seq << 32) | hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Polls until the slot carries `seq`; false after kQrSpinLimit polls or once `error` is up.
+// Polls until the slot carries `seq`; false after `spin_limit` polls or once `error` is up.
 template <typename T>
-__device__ __forceinline__ bool mail_fetch(const unsigned long long* slot, unsigned seq, const int* error, T* value) {
+__device__ __forceinline__ bool mail_fetch(const unsigned long long* slot, unsigned seq, const int* error,
+                                           unsigned spin_limit, T* value) {
   constexpr bool WIDE = sizeof(T) == 8;
   unsigned spins = 0;
   for (;;) {
@@ -122,7 +123,7 @@ __device__ __forceinline__ bool mail_fetch(const unsigned long long* slot, unsig
       return true;
     }
     ++spins;
-    if (spins > kQrSpinLimit) return false;
+    if (spins > spin_limit) return false;
     if ((spins & 63u) == 0 && __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
     __builtin_amdgcn_s_sleep(1);
   }
@@ -133,14 +134,14 @@ __device__ __forceinline__ bool mail_fetch(const unsigned long long* slot, unsig
 // Returns false if a message did not arrive; `s_fail` and `s_x` are shared scratch.
 template <typename T>
 __device__ __forceinline__ bool mail_gather(const unsigned long long* mail, int nwg, unsigned seq, int* error,
-                                            T* s_w, T* s_x, int* s_fail, T* sum, T* extra) {
+                                            unsigned spin_limit, T* s_w, T* s_x, int* s_fail, T* sum, T* extra) {
   const int tid = threadIdx.x;
   T v = T(0);
   bool ok = true;
-  if (tid < nwg) ok = mail_fetch<T>(mail + 2 * tid, seq, error, &v);
+  if (tid < nwg) ok = mail_fetch<T>(mail + 2 * tid, seq, error, spin_limit, &v);
   if (tid == 255) {
     T x = T(0);
-    ok = mail_fetch<T>(mail + 2 * kTrdMaxWg, seq, error, &x);
+    ok = mail_fetch<T>(mail + 2 * kTrdMaxWg, seq, error, spin_limit, &x);
     *s_x = x;
   }
   if (!ok) {
@@ -181,7 +182,8 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
                                                          T* __restrict__ t_part, int n_t_part,
                                                          T* __restrict__ dot_part, T* __restrict__ tau,
                                                          T* __restrict__ d, T* __restrict__ e,
-                                                         unsigned long long* mail, unsigned seq, int* error) {
+                                                         unsigned long long* mail, unsigned seq, int* error,
+                                                         unsigned spin_limit) {
   constexpr int NB = kTrdNb;
   __shared__ T s_t[2 * NB];
   __shared__ T s_t4[4][2 * NB];
@@ -250,7 +252,7 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
     if (tid == 0) mail_post(mail_dot + 2 * wg, dot, seq);
     if (r == jn) mail_post(mail_dot + 2 * kTrdMaxWg, wv, seq);  // the unfinished W[jn, i]
     T total, w_jn_raw;
-    if (!mail_gather<T>(mail_dot, nwg, seq, error, s_w4, &s_x, &s_fail, &total, &w_jn_raw)) return;
+    if (!mail_gather<T>(mail_dot, nwg, seq, error, spin_limit, s_w4, &s_x, &s_fail, &total, &w_jn_raw)) return;
     alpha2 = T(-0.5) * tau[j] * total;
     w_jn_i = w_jn_raw + alpha2;  // v_j has its unit entry in row jn
   }
@@ -286,7 +288,7 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
   if (tid == 0) mail_post(mail_norm + 2 * wg, norm_part, seq);
   if (r == jn + 1) mail_post(mail_norm + 2 * kTrdMaxWg, a, seq);  // alpha
   T x2_total, alpha;
-  if (!mail_gather<T>(mail_norm, nwg, seq, error, s_w4, &s_x, &s_fail, &x2_total, &alpha)) return;
+  if (!mail_gather<T>(mail_norm, nwg, seq, error, spin_limit, s_w4, &s_x, &s_fail, &x2_total, &alpha)) return;
 
   // ---- B(jn): reflector, v, partial W^T v and V^T v ----
   T beta = alpha, tauv = T(0), scale = T(0);
@@ -336,15 +338,6 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
   __syncthreads();
   if (tid < 2 * NB)
     t_part[(int64_t)wg * 2 * NB + tid] = (s_red[0][tid] + s_red[1][tid]) + (s_red[2][tid] + s_red[3][tid]);
-}
-
-// d[0..n) <- NaN if a workgroup of trd_column_kernel gave up waiting: the eigenvalues then come
-// out as NaN instead of silently wrong.
-template <typename T>
-__global__ void trd_poison_on_error_kernel(T* __restrict__ d, int n, const int* __restrict__ error) {
-  if (*error == 0) return;
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) d[i] = T(NAN);
 }
 
 // Kernel C.  The trailing matrix (rows and columns o = j+1 .. n-1, only its lower triangle is
@@ -421,9 +414,12 @@ __global__ __launch_bounds__(256) void trd_symv_kernel(const T* __restrict__ A, 
 
 // Tridiagonalise A (n x n, lower triangle referenced; destroyed).  On exit d[0..n), e[0..n-1),
 // tau[0..n-1) and, below the first subdiagonal of A, the reflector vectors (implicit unit at
-// row j+1 of column j), as LAPACK sytrd('L') leaves them.
+// row j+1 of column j), as LAPACK sytrd('L') leaves them.  *ws.error is nonzero afterwards if a
+// workgroup of the column kernel gave up waiting for a message; the results are then unusable and
+// the caller has to make that visible.
 template <typename T>
-static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* e, T* tau, const TrdWorkspace<T>& ws) {
+static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* e, T* tau, const TrdWorkspace<T>& ws,
+                              unsigned spin_limit = kQrSpinLimit) {
   constexpr int NB = kTrdNb;
   const int64_t ldw = n;
   if (n == 1) {
@@ -443,7 +439,8 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
     // open the panel: A(p), B(p)
     int grid = (int)ceil_div64(n - p, 256);
     hipLaunchKernelGGL((trd_column_kernel<T>), dim3(grid), dim3(256), 0, s, A, lda, n, p, p - 1, 0, 1, ws.vc, ws.vc2,
-                       ws.w, ldw, ws.y_part, 0, ws.t_part, 0, ws.dot_part, tau, d, e, ws.mail, ++seq, ws.error);
+                       ws.w, ldw, ws.y_part, 0, ws.t_part, 0, ws.dot_part, tau, d, e, ws.mail, ++seq, ws.error,
+                       spin_limit);
     int t_parts = grid;  // grid of the launch that ran B for the current column
     int cols_done = 0, last_dot_parts = 0;
     for (int j = p; j < pe; ++j) {
@@ -457,7 +454,7 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
       const int do_next = (j + 1 < pe) ? 1 : 0;
       hipLaunchKernelGGL((trd_column_kernel<T>), dim3(grid), dim3(256), 0, s, A, lda, n, p, j, 1, do_next, ws.vc, ws.vc2,
                          ws.w, ldw, ws.y_part, nb, ws.t_part, t_parts, ws.dot_part, tau, d, e, ws.mail, ++seq,
-                         ws.error);
+                         ws.error, spin_limit);
       t_parts = grid;
       last_dot_parts = grid;
       cols_done = i + 1;
@@ -483,9 +480,6 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
       if (rc) return rc;
     }
   }
-  hipLaunchKernelGGL((trd_poison_on_error_kernel<T>), dim3((unsigned)ceil_div64(n, 256)), dim3(256), 0, s, d, n,
-                     ws.error);
-  SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
 

@@ -176,6 +176,40 @@ def test_qr_launch_per_column_panel_path(size, device):
         _native.call("soapmi_set_option", b"qr_persistent_max_workgroups", 129)
 
 
+def test_lost_messages_poison_the_result_instead_of_hanging(device):
+    """With no patience for another workgroup's message (spin limit 0) the persistent kernels leave
+    early; the outputs must then be NaN-poisoned or, if every message happened to be there at the
+    first poll, correct - never silently wrong - and the next call with the default limit is clean."""
+    from soap_tp_amd import _native
+    size = 700  # three workgroups of 256 rows
+    matrix = make_matrix(size, size, seed=SEED + 77)
+    symmetric = make_preconditioner(size, SEED + 78).double()
+    expected_q = oracle.householder_qr(matrix)
+    expected_values = torch.linalg.eigvalsh(symmetric)
+
+    def run():
+        factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+        ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
+        a = column_major(symmetric, device)
+        values = torch.empty(size, dtype=torch.float64, device=device)
+        vectors = torch.empty(size, size, dtype=torch.float64, device=device).T
+        _native.call("soapmi_eigh_f64", a.data_ptr(), values.data_ptr(), vectors.data_ptr(), size, a.stride(1),
+                     vectors.stride(1), 0, 0, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        return factor.cpu(), values.cpu()
+
+    try:
+        _native.call("soapmi_set_option", b"message_spin_limit", 0)
+        factor, values = run()
+    finally:
+        _native.call("soapmi_set_option", b"message_spin_limit", 1 << 22)
+    assert torch.isnan(factor).any() or relative_l2(factor, expected_q) <= 5e-5
+    assert torch.isnan(values).all() or relative_l2(values, expected_values) <= 1e-12
+    factor, values = run()
+    assert relative_l2(factor, expected_q) <= 5e-5
+    assert relative_l2(values, expected_values) <= 1e-12
+
+
 def test_argsort_ties_and_large(device):
     from soap_tp_amd import _native
     for count in (1, 2, 33, 4096, 16384, 20000):
