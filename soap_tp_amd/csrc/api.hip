@@ -202,8 +202,13 @@ int soapmi_gram_ema_f32(const float* g, int64_t rows, int64_t cols, int64_t ldg,
   // right = G^T G : row-major -> S S^T (0, 1)               ; col-major -> S^T S (1, 0)
   const bool stts = (side == 0) == (g_row_major != 0);
   const int ta = stts ? 1 : 0, tb = stts ? 0 : 1;
-  GemmProblem<float> prob = make_problem<float>(ta, tb, (int)n, (int)n, (int)k, g, ldg, g, ldg, true);
   EpiEmaLower<float> epi{p, ldp, 1.0f - beta, mirror};
+  if (prefer_small_tile<float>(n, n, true)) {
+    using Small = SmallTile<float>::type;
+    GemmProblem<float> prob = make_problem<float, Small>(ta, tb, (int)n, (int)n, (int)k, g, ldg, g, ldg, true);
+    return launch_gemm<float, EpiEmaLower<float>, Small>((hipStream_t)stream, prob, epi, 1);
+  }
+  GemmProblem<float> prob = make_problem<float>(ta, tb, (int)n, (int)n, (int)k, g, ldg, g, ldg, true);
   return launch_gemm<float>((hipStream_t)stream, prob, epi, 1);
 }
 
@@ -297,9 +302,15 @@ int soapmi_rotate_adam_rotate_f32(const float* gradient, int64_t ldg, float* upd
   if (rc) return rc;
   // 2. U = adam(H QR): the rotated gradient stays in the accumulators.
   {
-    GemmProblem<float> prob = make_problem<float>(0, 0, m, n, n, h, rows, qr, ldqr, false);
     EpiAdam epi{momentum, variance, u, ldm, ldv, rows, sc};
-    rc = launch_gemm<float>(s, prob, epi, 1);
+    if (prefer_small_tile<float>(m, n, false)) {
+      using Small = SmallTile<float>::type;
+      GemmProblem<float> prob = make_problem<float, Small>(0, 0, m, n, n, h, rows, qr, ldqr, false);
+      rc = launch_gemm<float, EpiAdam, Small>(s, prob, epi, 1);
+    } else {
+      GemmProblem<float> prob = make_problem<float>(0, 0, m, n, n, h, rows, qr, ldqr, false);
+      rc = launch_gemm<float>(s, prob, epi, 1);
+    }
     if (rc) return rc;
   }
   // 3. H = QL U
