@@ -221,6 +221,47 @@ def run_layer(device, steps=30, rank=64):
             "initialisation_ms": init_ms, "plain_step_mfma_flops": flops}
 
 
+def hbm_stages(rows, columns, device, repeats=10):
+    """The bandwidth-bound kernels of the path, each timed alone with HIP events over `repeats` launches:
+    achieved GB/s over their algorithmic bytes against the 8 TB/s HBM peak."""
+    from soap_tp_amd.ops import (adam_update, allocate_2d_block_cyclic, permute_2d_block_cyclic_,
+                                 redistribute_tp_shard_to_2d_block_cyclic)
+
+    def timed(function):
+        function()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        for _ in range(repeats):
+            function()
+        end.record()
+        torch.cuda.synchronize()
+        return begin.elapsed_time(end) / repeats
+
+    shape = (rows, columns)
+    gradient = allocate_2d_block_cyclic(shape, 128, GRID, device=device)
+    gradient.normal_()
+    momentum = allocate_2d_block_cyclic(shape, 128, GRID, device=device)
+    variance = allocate_2d_block_cyclic(shape, 128, GRID, device=device)
+    row_major = torch.randn(rows, columns, device=device)
+    row_order = torch.randperm(rows, device=device)
+    column_order = torch.randperm(columns, device=device)
+    stages = {
+        "adam_kernel": (24.0 * rows * columns,
+                        lambda: adam_update(gradient, momentum, variance, 3, 0.95, 0.95, 1e-8)),
+        "layout_copy": (8.0 * rows * columns,
+                        lambda: redistribute_tp_shard_to_2d_block_cyclic(row_major, shape, 128, GRID, shard_dim=1)),
+        "variance_permute": (16.0 * rows * columns,  # gather into a temporary, copy back
+                             lambda: permute_2d_block_cyclic_(variance, shape, row_order, column_order, 128, GRID,
+                                                              validate=False)),
+    }
+    result = {}
+    for name, (nbytes, function) in stages.items():
+        ms = timed(function)
+        rate = nbytes / (ms * 1e-3) / 1e9
+        result[name] = {"bytes": nbytes, "ms": ms, "GB/s": rate, "frac_of_hbm_peak": rate / HBM_PEAK_GBS}
+    return result
+
+
 def calibration_copies(rows, columns, count, device):
     """Row-major to column-major copies of a rows x columns fp32 matrix through the library."""
     from soap_tp_amd.ops import redistribute_tp_shard_to_2d_block_cyclic
@@ -332,6 +373,7 @@ def main():
                 "initialisation_call_ms": run["init_ms"], "step_mfma_stages_tflops": flops / (plain * 1e-3) / 1e12,
             }
         line["other_shapes"] = others
+    line["hbm_stages"] = hbm_stages(rows, columns, device)
     if args.layer:
         line["layer"] = run_layer(device)
     if not args.no_cpu_baseline:
