@@ -6,7 +6,7 @@
 A "step" is one ``soap_step`` call on a synthetic low-rank-plus-noise gradient that is already
 resident in HBM.  The warm-up contains the initialising call (Gram matrices + both eigensolves) and,
 by default, ten more steps including one basis refresh, so that the timed region is the
-steady-state schedule of BASELINE's configuration: K steps with a refresh every 10.  One JSON line
+steady-state schedule of the benchmark configuration: K steps with a refresh every 10.  One JSON line
 is printed; ``value`` is K divided by the time of the timed region, taken with HIP events on the
 stream the kernels run on and bracketed by device synchronisations.
 

@@ -1,7 +1,7 @@
 """End-to-end parity of ``soap_step`` on the GPU against the CPU oracle and the golden trajectory
 of the original optimizer, restating tests/unit/test_soap.py of the reference for one rank
 (10 iterations, refresh every 2, betas 0.75 / 0.8 / 0.9, eps 1e-6, N(0, 2) gradients, block 2),
-then BASELINE's first configuration and size-independent properties at the benchmark sizes.
+then the benchmark's first configuration (1024 x 1024) and size-independent properties at the benchmark sizes.
 
 Bar: relative Frobenius error <= 1e-4 on updates, moments and Gram matrices (float32 path).
 Where eigenvectors are not determined to working precision by the data (clusters of nearly equal
@@ -203,7 +203,7 @@ def test_profile_lines(device, monkeypatch, capsys):
     assert first["impl"] == "tp" and first["shape"] == [8, 8] and len(first["values"]) == 64
 
 
-# ---- BASELINE configuration 1: 1024 x 1024, rank 32 low-rank-plus-noise, 20 steps, refresh 10 ----
+# ---- benchmark configuration 1: 1024 x 1024, rank 32 low-rank-plus-noise, 20 steps, refresh 10 ----
 def test_baseline_config_1024(device, monkeypatch):
     rows = columns = 1024
     kwargs = dict(preconditioner_beta=0.95, beta1=0.95, beta2=0.95, eps=1e-8, basis_refresh_interval=10)
