@@ -200,6 +200,8 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
 // launch's starting value and clears the mailboxes before the first panel), mailboxes alternate
 // between two sets by column parity: a workgroup writes column c+2 only after it has read every
 // workgroup's column c+1, which those wrote after they had read column c.
+// Besides A the kernel writes the panel's reflectors in clean form (unit diagonal, zeros above) to
+// vout, the operand of the block-reflector products.
 // Requirements: all workgroups of the launch are resident at the same time (the host launches at
 // most kQrPersistentMaxWg of them, one per CU).  Waiting is bounded: a thread that does not see a
 // word arrive within `spin_limit` polls (kQrSpinLimit unless the caller lowers it) raises `error`, and every workgroup that sees the flag or
@@ -243,7 +245,8 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
                                                                   int pe, unsigned long long* part,
                                                                   unsigned long long* piv, float* __restrict__ tau,
                                                                   unsigned seq_base, int* error, int nwg,
-                                                                  unsigned spin_limit) {
+                                                                  unsigned spin_limit, float* __restrict__ vout,
+                                                                  int64_t ldv, int vrow0) {
   using T = float;
   constexpr int NB = kQrNb;
   __shared__ T s_tc[NB];
@@ -259,6 +262,11 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
   const int nbw = pe - p;
   const bool live = r < n;
   if (tid == 0) s_fail = 0;
+  // vout (rows vrow0.., one column per panel column) receives the reflectors in clean form: zeros
+  // above the unit diagonal, including the vrow0 - p ... rows above the panel that no thread owns
+  if (wg == 0) {
+    for (int t = tid; t < (p - vrow0) * nbw; t += 256) vout[t % (p - vrow0) + (int64_t)(t / (p - vrow0)) * ldv] = T(0);
+  }
 
   T a[NB];  // a[k] = A[r, j + k] for the current column j: the row is shifted left after each column
 #pragma unroll
@@ -358,7 +366,10 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
         tau[j] = tauv;
       }
     }
-    if (live) A[r + (int64_t)j * lda] = a[0];  // column j is final
+    if (live) {
+      A[r + (int64_t)j * lda] = a[0];  // column j is final
+      vout[(r - vrow0) + (int64_t)c * ldv] = (r > j) ? a[0] : (r == j ? T(1) : T(0));
+    }
 #pragma unroll
     for (int k = 0; k + 1 < NB; ++k) a[k] = a[k + 1];
     a[NB - 1] = T(0);
@@ -384,50 +395,67 @@ __global__ void extract_v_kernel(const T* __restrict__ A, int64_t lda, int nrows
   }
 }
 
+// Value of `v` in lane `LANE` (a compile-time constant) as a wavefront-uniform scalar.
+template <int LANE>
+__device__ __forceinline__ float lane_value(float v) {
+  return __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)__float_as_uint(v), LANE));
+}
+template <int LANE>
+__device__ __forceinline__ double lane_value(double v) {
+  const int lo = __builtin_amdgcn_readlane(__double2loint(v), LANE);
+  const int hi = __builtin_amdgcn_readlane(__double2hiint(v), LANE);
+  return __hiloint2double(hi, lo);
+}
+
+// Column I of the factor, for I = 0 .. 31 by recursion: lane k holds row k of T in t[] and row k of
+// G in g[]; T[0:I, I] = -tau_I T[0:I, 0:I] G[0:I, I], where G[l, I] is fetched from lane l's
+// register and T[k, l] is zero below the diagonal, so every lane runs the same I multiply-adds.
+template <typename T, int I>
+struct LarftColumn {
+  template <int L>
+  static __device__ __forceinline__ T dot(const T (&t)[32], const T& g_i) {
+    if constexpr (L < 0) {
+      return T(0);
+    } else {
+      return dot<L - 1>(t, g_i) + t[L] * lane_value<L>(g_i);
+    }
+  }
+  static __device__ __forceinline__ void run(T (&t)[32], const T (&g)[32], T tau_k, int k) {
+    if constexpr (I > 0) LarftColumn<T, I - 1>::run(t, g, tau_k, k);
+    const T tau_i = lane_value<I>(tau_k);
+    const T acc = dot<I - 1>(t, g[I]);
+    t[I] = (k < I) ? -tau_i * acc : (k == I ? tau_i : T(0));
+  }
+};
+
 // Compact-WY factor of up to 32 reflectors: T upper triangular with H_0 ... H_{w-1} = I - V T V^T,
 // from G = V^T V (LAPACK larft, forward / columnwise).  One wavefront per 32-wide diagonal block:
 // blockIdx.x selects the block (G, tau and T advance along the diagonal), so the diagonal blocks
-// of a wider factor are built by one launch.  Column i needs the finished columns 0..i-1; the
-// inner product is unrolled four ways to overlap LDS latency.
+// of a wider factor are built by one launch.  Everything stays in registers: the recursion over
+// the columns is unrolled at compile time and values cross lanes as scalars (v_readlane).
+// Reflectors beyond the block's width count as tau = 0, which leaves their rows and columns zero.
 template <typename T>
 __global__ __launch_bounds__(64) void larft32_kernel(const T* __restrict__ G, int ldg, const T* __restrict__ tau,
                                                       int nbw, T* __restrict__ Tm, int ldt) {
-  __shared__ T t[32][33];
-  __shared__ T g[32][33];
   const int b = blockIdx.x;
   const int w = min(32, nbw - 32 * b);
   G += (int64_t)32 * b * (ldg + 1);
   Tm += (int64_t)32 * b * (ldt + 1);
   tau += 32 * b;
-  const int k = threadIdx.x;
-  if (k < 32) {
-    for (int c = 0; c < 32; ++c) {
-      t[k][c] = T(0);
-      g[k][c] = (k < w && c < w) ? G[k + c * ldg] : T(0);
-    }
+  const int k = threadIdx.x;  // lanes 32..63 carry zeros
+  T t[32], g[32];
+#pragma unroll
+  for (int c = 0; c < 32; ++c) {
+    t[c] = T(0);
+    g[c] = (k < w && c < w) ? G[k + c * ldg] : T(0);
   }
-  __syncthreads();
-  for (int i = 0; i < w; ++i) {
-    const T ti = tau[i];
-    T s0 = T(0), s1 = T(0), s2 = T(0), s3 = T(0);
-    if (k < i) {
-      int l = k;
-      for (; l + 4 <= i; l += 4) {
-        s0 += t[k][l] * g[l][i];
-        s1 += t[k][l + 1] * g[l + 1][i];
-        s2 += t[k][l + 2] * g[l + 2][i];
-        s3 += t[k][l + 3] * g[l + 3][i];
-      }
-      for (; l < i; ++l) s0 += t[k][l] * g[l][i];
-    }
-    const T s = -ti * ((s0 + s1) + (s2 + s3));
-    __syncthreads();
-    if (k < i) t[k][i] = s;
-    if (k == i) t[i][i] = ti;
-    __syncthreads();
+  const T tau_k = (k < w) ? tau[k] : T(0);
+  LarftColumn<T, 31>::run(t, g, tau_k, k);
+  if (k < w) {
+#pragma unroll
+    for (int c = 0; c < 32; ++c)
+      if (c < w) Tm[k + c * ldt] = t[c];
   }
-  if (k < w)
-    for (int c = 0; c < w; ++c) Tm[k + c * ldt] = t[k][c];
 }
 
 // Fills the diagonal of Q with NaN if the error flag is set.
@@ -635,15 +663,20 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     T* Tm = ws.t_all + (size_t)bi * OB * OB;
     hipLaunchKernelGGL((fill_zero_kernel<T>), dim3(OB * OB / 256), dim3(256), 0, s, Tm, OB * OB);
     int inner_done = 0;
+    bool v_written = true;  // the panel kernels leave the block's reflectors in ws.br.v
     for (int p = P; p < PE; p += NB) {
       const int pe = std::min(PE, p + NB), nbw = pe - p;
       const int rows = n - p;
       const int nwg = (int)ceil_div64(rows, 256);
       T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
       T* piv[2] = {ws.piv, ws.piv + NB};
+      // this panel's reflectors inside the outer block's n x 128 buffer (origin: row P, column P)
+      BlockReflectorWs<T> inner = ws.br;
+      inner.v = ws.br.v + (p - P) + (int64_t)(p - P) * ldv;
       if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
-                           ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit);
+                           ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
+                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P);
         seq_base += (unsigned)nbw;
       } else {
         for (int j = p - 1; j < pe; ++j) {
@@ -651,22 +684,23 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
           hipLaunchKernelGGL((qr_panel_step_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, j, part[in],
                              piv[in], part[out], piv[out], ws.tau, nwg);
         }
+        v_written = false;
       }
       SOAPMI_LAUNCH_CHECK();
       if (pe < PE) {  // the panel's reflectors act on the rest of the outer block only
         T* Tin = Tm + (int64_t)(p - P) * (OB + 1);  // diagonal block of the outer factor
-        launch_extract_v<T>(s, A, lda, rows, p, p, nbw, ws.br.v, ldv);
-        rc = gram_of_v<T>(s, ws.br, rows, nbw, ldv);
+        if (!v_written) launch_extract_v<T>(s, A, lda, rows, p, p, nbw, inner.v, ldv);
+        rc = gram_of_v<T>(s, inner, rows, nbw, ldv);
         if (rc) return rc;
-        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(64), 0, s, ws.br.gram, OB, ws.tau + p, nbw, Tin, OB);
+        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(64), 0, s, inner.gram, OB, ws.tau + p, nbw, Tin, OB);
         SOAPMI_LAUNCH_CHECK();
-        rc = apply_block_reflector<T>(s, ws.br, Tin, true, rows, nbw, PE - pe, ldv, A + p + (int64_t)pe * lda, lda);
+        rc = apply_block_reflector<T>(s, inner, Tin, true, rows, nbw, PE - pe, ldv, A + p + (int64_t)pe * lda, lda);
         if (rc) return rc;
         ++inner_done;
       }
     }
     const int rows = n - P;
-    launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
+    if (!v_written) launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
     rc = gram_of_v<T>(s, ws.br, rows, obw, ldv);
     if (rc) return rc;
     rc = assemble_t_factor<T>(s, ws.br, obw, ws.tau + P, Tm, inner_done);
