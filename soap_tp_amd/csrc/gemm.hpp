@@ -529,6 +529,26 @@ static inline int gemm(hipStream_t stream, int transA, int transB, int M, int N,
   return launch_gemm<T, EpiStore<T>, Cfg>(stream, p, ep, 1);
 }
 
+// op(A) op(B) cut into K slices whose partial products stay unreduced in `partials` (slice z at
+// partials + z * M * N, column-major with leading dimension M), for consumers that sum the slices
+// themselves.  *splits_out receives the number of slices written (at least 1).
+template <typename T, class Cfg = typename DefaultTile<T>::type>
+static inline int gemm_to_partials(hipStream_t stream, int transA, int transB, int M, int N, int K, const T* A,
+                                   int64_t lda, const T* B, int64_t ldb, int k_splits, T* partials, int* splits_out) {
+  *splits_out = 1;
+  if (M <= 0 || N <= 0) return kOk;
+  GemmProblem<T> p = make_problem<T, Cfg>(transA, transB, M, N, K, A, lda, B, ldb, false);
+  int splits = 1;
+  if (k_splits > 1 && K > Cfg::BK) {
+    const int64_t slabs = ceil_div64(K, Cfg::BK);
+    p.k_chunk = (int)(ceil_div64(slabs, k_splits) * Cfg::BK);
+    splits = (int)ceil_div64(K, p.k_chunk);
+  }
+  *splits_out = splits;
+  EpiPartial<T> ep{partials, (int64_t)M, (int64_t)M * N};
+  return launch_gemm<T, EpiPartial<T>, Cfg>(stream, p, ep, splits);
+}
+
 // Square product restricted to the tiles on or below the diagonal of C (n x n): entries of C above
 // the diagonal tiles are neither read nor written; inside diagonal tiles the whole tile is updated.
 template <typename T, class Cfg = typename DefaultTile<T>::type>

@@ -434,27 +434,54 @@ struct LarftColumn {
 // of a wider factor are built by one launch.  Everything stays in registers: the recursion over
 // the columns is unrolled at compile time and values cross lanes as scalars (v_readlane).
 // Reflectors beyond the block's width count as tau = 0, which leaves their rows and columns zero.
+// G may arrive as `splits` unreduced split-K slices (`slab` elements apart), summed while loading.
 template <typename T>
-__global__ __launch_bounds__(64) void larft32_kernel(const T* __restrict__ G, int ldg, const T* __restrict__ tau,
-                                                      int nbw, T* __restrict__ Tm, int ldt) {
+__global__ __launch_bounds__(128) void larft32_kernel(const T* __restrict__ G, int ldg, int splits, int64_t slab,
+                                                       const T* __restrict__ tau, int nbw, T* __restrict__ Tm,
+                                                       int ldt) {
+  __shared__ T s_g[4][32][33];
   const int b = blockIdx.x;
   const int w = min(32, nbw - 32 * b);
   G += (int64_t)32 * b * (ldg + 1);
   Tm += (int64_t)32 * b * (ldt + 1);
   tau += 32 * b;
-  const int k = threadIdx.x;  // lanes 32..63 carry zeros
+  const int k = threadIdx.x & 31, zg = threadIdx.x >> 5;
   T t[32], g[32];
+  // slices z = zg, zg + 4, ... are summed by slice group zg (128 threads = 4 groups), the groups then
+  // in a fixed order
 #pragma unroll
-  for (int c = 0; c < 32; ++c) {
-    t[c] = T(0);
-    g[c] = (k < w && c < w) ? G[k + c * ldg] : T(0);
-  }
-  const T tau_k = (k < w) ? tau[k] : T(0);
-  LarftColumn<T, 31>::run(t, g, tau_k, k);
+  for (int c = 0; c < 32; ++c) g[c] = T(0);
   if (k < w) {
+    for (int z = zg; z < splits; z += 4) {
+      const T* slice = G + (int64_t)z * slab + k;
+#pragma unroll
+      for (int c = 0; c < 32; ++c) g[c] += (c < w) ? slice[c * ldg] : T(0);
+    }
+  }
+  if (splits > 1) {
+#pragma unroll
+    for (int c = 0; c < 32; ++c) s_g[zg][k][c] = g[c];
+    __syncthreads();
+    if (zg == 0) {
+#pragma unroll
+      for (int c = 0; c < 32; ++c)
+        g[c] = (s_g[0][k][c] + s_g[1][k][c]) + (s_g[2][k][c] + s_g[3][k][c]);
+    }
+  }
+  if (threadIdx.x >= 64) return;  // the recursion runs in the first wavefront; its lanes 32..63 carry zeros
+  const int lane = threadIdx.x;
+  if (lane >= 32) {
+#pragma unroll
+    for (int c = 0; c < 32; ++c) g[c] = T(0);
+  }
+#pragma unroll
+  for (int c = 0; c < 32; ++c) t[c] = T(0);
+  const T tau_k = (lane < w) ? tau[lane] : T(0);
+  LarftColumn<T, 31>::run(t, g, tau_k, lane);
+  if (lane < w) {
 #pragma unroll
     for (int c = 0; c < 32; ++c)
-      if (c < w) Tm[k + c * ldt] = t[c];
+      if (c < w) Tm[lane + c * ldt] = t[c];
   }
 }
 
@@ -484,7 +511,7 @@ __global__ void orgqr_panel_fix_kernel(T* __restrict__ Q, int64_t ldq, int p, in
 }
 
 // ---- block reflectors ------------------------------------------------------------------------
-constexpr int kBrMax = 128;   // widest block reflector (outer block of the QR, back-transformation)
+constexpr int kBrMax = 256;   // widest block reflector (outer block of the QR, back-transformation)
 constexpr int kBrSplits = 8;  // split-K slices of the tall-skinny products
 
 template <typename T>
@@ -519,8 +546,8 @@ static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws
   using Skinny = typename SkinnyTile<T>::type;
   const int blocks = (int)ceil_div64(nbw, 32);
   if (first_block < blocks) {
-    hipLaunchKernelGGL((larft32_kernel<T>), dim3(blocks - first_block), dim3(64), 0, s,
-                       ws.gram + (int64_t)32 * first_block * (kBrMax + 1), kBrMax, tau + 32 * first_block,
+    hipLaunchKernelGGL((larft32_kernel<T>), dim3(blocks - first_block), dim3(128), 0, s,
+                       ws.gram + (int64_t)32 * first_block * (kBrMax + 1), kBrMax, 1, (int64_t)0, tau + 32 * first_block,
                        nbw - 32 * first_block, Tm + (int64_t)32 * first_block * (kBrMax + 1), kBrMax);
     SOAPMI_LAUNCH_CHECK();
   }
@@ -544,6 +571,36 @@ static inline int split_count(int64_t tiles, int rows, int M, int N, int64_t ldv
   const int64_t capacity = (int64_t)kBrSplits * kBrMax * ldv / std::max<int64_t>(1, (int64_t)M * N);
   splits = std::min<int64_t>(splits, std::min<int64_t>(capacity, 64));
   return (int)std::max<int64_t>(splits, 1);
+}
+
+// W2 (M x N, ld ldw2) = op(T) * (sum of the split-K slices of W), M <= 32: the middle product of a
+// 32-wide block reflector, taking V^T C straight from the slices (slice z at part + z * slab,
+// leading dimension M).  256 threads own 32 rows x 2 columns x 4 groups of slices.
+template <typename T>
+__global__ __launch_bounds__(256) void reflector_w2_kernel(const T* __restrict__ part, int splits, int64_t slab, int M,
+                                                           int N, const T* __restrict__ Tm, int ldt, int trans_t,
+                                                           T* __restrict__ W2, int ldw2) {
+  __shared__ T s_t[32][33];
+  __shared__ T s_w[2][4][33];
+  const int tid = threadIdx.x, l = tid & 31, zg = (tid >> 5) & 3, cc = tid >> 7;
+  const int c = blockIdx.x * 2 + cc;
+  for (int q = tid >> 5; q < 32; q += 8) {  // s_t[a][b] = op(T)[a, b]
+    const T v = (l < M && q < M) ? Tm[l + q * ldt] : T(0);  // T[l, q]
+    if (trans_t) s_t[q][l] = v;
+    else s_t[l][q] = v;
+  }
+  T sum = T(0);
+  if (l < M && c < N)
+    for (int z = zg; z < splits; z += 4) sum += part[(int64_t)z * slab + l + (int64_t)c * M];
+  s_w[cc][zg][l] = sum;
+  __syncthreads();
+  if (zg == 0 && l < M && c < N) {
+    T acc = T(0);
+#pragma unroll
+    for (int q = 0; q < 32; ++q)
+      acc += s_t[l][q] * ((s_w[cc][0][q] + s_w[cc][1][q]) + (s_w[cc][2][q] + s_w[cc][3][q]));
+    W2[l + (int64_t)c * ldw2] = acc;
+  }
 }
 
 template <typename T>
@@ -580,9 +637,13 @@ static inline int apply_block_reflector(hipStream_t s, const BlockReflectorWs<T>
   const int splits = split_count(tiles, rows, nbw, nc, ldv);
   int rc;
   if (skinny) {
-    rc = gemm<T, Skinny>(s, 1, 0, nbw, nc, rows, T(1), ws.v, ldv, C, ldc, T(0), ws.w, kBrMax, splits, ws.splitk);
+    int slices = 1;
+    rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, nc, rows, ws.v, ldv, C, ldc, splits, ws.splitk, &slices);
     if (rc) return rc;
-    rc = gemm<T, Skinny>(s, transT ? 1 : 0, 0, nbw, nc, nbw, T(1), Tm, kBrMax, ws.w, kBrMax, T(0), ws.w2, kBrMax);
+    hipLaunchKernelGGL((reflector_w2_kernel<T>), dim3((unsigned)ceil_div64(nc, 2)), dim3(256), 0, s, ws.splitk, slices,
+                       (int64_t)nbw * nc, nbw, nc, Tm, kBrMax, transT ? 1 : 0, ws.w2, kBrMax);
+    SOAPMI_LAUNCH_CHECK();
+    rc = kOk;
   } else {
     rc = gemm<T>(s, 1, 0, nbw, nc, rows, T(1), ws.v, ldv, C, ldc, T(0), ws.w, kBrMax, splits, ws.splitk);
     if (rc) return rc;
@@ -690,9 +751,13 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       if (pe < PE) {  // the panel's reflectors act on the rest of the outer block only
         T* Tin = Tm + (int64_t)(p - P) * (OB + 1);  // diagonal block of the outer factor
         if (!v_written) launch_extract_v<T>(s, A, lda, rows, p, p, nbw, inner.v, ldv);
-        rc = gram_of_v<T>(s, inner, rows, nbw, ldv);
+        int slices = 1;  // V^T V stays in split-K slices; the factor kernel sums them while loading
+        rc = gemm_to_partials<T, typename SkinnyTile<T>::type>(s, 1, 0, nbw, nbw, rows, inner.v, ldv, inner.v, ldv,
+                                                               split_count(1, rows, nbw, nbw, ldv), inner.splitk,
+                                                               &slices);
         if (rc) return rc;
-        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(64), 0, s, inner.gram, OB, ws.tau + p, nbw, Tin, OB);
+        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(128), 0, s, inner.splitk, nbw, slices,
+                           (int64_t)nbw * nbw, ws.tau + p, nbw, Tin, OB);
         SOAPMI_LAUNCH_CHECK();
         rc = apply_block_reflector<T>(s, inner, Tin, true, rows, nbw, PE - pe, ldv, A + p + (int64_t)pe * lda, lda);
         if (rc) return rc;
