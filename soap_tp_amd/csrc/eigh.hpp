@@ -4,7 +4,6 @@
 // (src/soap_tp/csrc/elpa_bindings.cpp:149,165); eigenvalues come back ascending.
 #pragma once
 #include "common.hpp"
-#include "elementwise.hpp"
 #include "gemm.hpp"
 #include "qr.hpp"
 #include "stedc.hpp"
