@@ -61,7 +61,7 @@ class StepTimer:
         return event
 
 
-def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True):
+def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True, shard_dim=1):
     import soap_tp_amd
     from soap_tp_amd import soap as soap_module
     from soap_tp_amd.ops import (refresh_bases_and_transport_optimizer_state_,
@@ -72,7 +72,7 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True):
     gradients = [device_low_rank_plus_noise(rows, columns, rank, 42 + i, device) for i in range(pool_size)]
     torch.cuda.synchronize()
     state = {}
-    kwargs = dict(global_shape=shape, shard_dim=1, block_size=128, process_grid_shape=GRID, **HYPER)
+    kwargs = dict(global_shape=shape, shard_dim=shard_dim, block_size=128, process_grid_shape=GRID, **HYPER)
 
     init_start = time.perf_counter()
     soap_tp_amd.soap_step(gradients[0], state, **kwargs)
@@ -98,11 +98,11 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True):
                                                HYPER["eps"])
             t1 = timer.mark()
             update_left_preconditioner_2d_block_cyclic_(gradient, state["left_preconditioner"],
-                                                        HYPER["preconditioner_beta"], 128, GRID, shard_dim=1,
+                                                        HYPER["preconditioner_beta"], 128, GRID, shard_dim=shard_dim,
                                                         mirror=False)
             update_right_preconditioner_2d_block_cyclic_(gradient, state["right_preconditioner"],
-                                                         HYPER["preconditioner_beta"], 128, GRID, shard_dim=1,
-                                                         mirror=False)
+                                                         HYPER["preconditioner_beta"], 128, GRID,
+                                                         shard_dim=shard_dim, mirror=False)
             t2 = timer.mark()
             refreshed = step % interval == 0
             if refreshed:
@@ -284,6 +284,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=11)
     parser.add_argument("--shape", type=parse_shape, default=(4096, 11008))
     parser.add_argument("--rank", type=int, default=128)
+    parser.add_argument("--shard-dim", type=int, default=1, choices=(0, 1),
+                        help="shard_dim passed to the step (same mathematics on one rank; the reference's two Gram "
+                             "code paths)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-other-shapes", action="store_true")
     parser.add_argument("--cpu-full-init", action="store_true",
@@ -309,7 +312,7 @@ def main():
 
     if args.calibration_copies > 0:
         calibration_copies(rows, columns, args.calibration_copies, device)
-    main_run = run_schedule(args.shape, args.rank, args.steps, args.warmup, device)
+    main_run = run_schedule(args.shape, args.rank, args.steps, args.warmup, device, shard_dim=args.shard_dim)
     ms_per_step = main_run["total_ms"] / args.steps
     rotation_flops = 4.0 * rows * columns * (rows + columns)
     gram_flops = 1.0 * rows * columns * (rows + columns)
@@ -330,7 +333,8 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"{rows}x{columns} fp32 parameter, rank-{args.rank} low-rank-plus-noise gradients "
-                        f"(log-uniform spectrum 1e-4..1e-1, noise std 1e-4), world_size 1, block_size 128, "
+                        f"(log-uniform spectrum 1e-4..1e-1, noise std 1e-4), world_size 1, shard_dim {args.shard_dim}, "
+                        f"block_size 128, "
                         f"refresh every {HYPER['basis_refresh_interval']} steps, beta1=beta2=shampoo_beta=0.95, "
                         "eps=1e-8, basis_implementation=elpa (fp64 eigensolve)",
             "schedule": f"{args.warmup} warm-up calls (initialisation + {args.warmup - 1} steps), then {args.steps} "
