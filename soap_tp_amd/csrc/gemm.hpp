@@ -128,6 +128,20 @@ struct GemmTile {
   static_assert((BK * BM / VW) % NT == 0 && (BK * BN / VW) % NT == 0, "loader tiling");
 };
 
+// Which 16-byte piece of a k-contiguous operand slab vector index v handles: KV pieces along k for
+// each x.  Sixteen consecutive lanes take sixteen consecutive x at one k piece, the next sixteen
+// lanes the next k piece: the transposing LDS stores S[k][x] of 32 lanes then fall into 32 distinct
+// banks (with v -> (v / KV, v % KV) two k pieces 2*KV rows apart shared their banks).  Global
+// loads do not care: a wavefront's load covers the same set of 64-byte segments either way.
+template <int KV>
+__device__ __forceinline__ int kcontig_x(int v) {
+  return 16 * (v / (16 * KV)) + (v & 15);
+}
+template <int KV>
+__device__ __forceinline__ int kcontig_kv(int v) {
+  return (v >> 4) % KV;
+}
+
 // Load one K-slab of an operand into registers.  X is the non-K extent (M for A, N for B).
 // xcontig: element (x, k) lives at base[x + k*ld]; otherwise at base[k + x*ld].
 template <typename T, int BX, int BK, int NT, int NV>
@@ -157,7 +171,7 @@ __device__ __forceinline__ void load_slab(T (&reg)[NV][Vec16<T>::W], const T* __
         for (int e = 0; e < VW; ++e) reg[i][e] = (gx + e < X && gk < kend) ? p[e] : T(0);
       }
     } else {
-      int x = v / (BK / VW), kv = v % (BK / VW);
+      int x = kcontig_x<BK / VW>(v), kv = kcontig_kv<BK / VW>(v);
       int gx = x0 + x, gk = k0 + kv * VW;
       const T* p = base + gk + (int64_t)gx * ld;
       if (vec) {
@@ -193,7 +207,7 @@ __device__ __forceinline__ void store_slab(T* __restrict__ S, const T (&reg)[NV]
       for (int e = 0; e < VW; ++e) tp[e] = reg[i][e];
       *reinterpret_cast<V*>(S + k * STRIDE + xv * VW) = t;
     } else {
-      int x = v / (BK / VW), kv = v % (BK / VW);
+      int x = kcontig_x<BK / VW>(v), kv = kcontig_kv<BK / VW>(v);
 #pragma unroll
       for (int e = 0; e < VW; ++e) S[(kv * VW + e) * STRIDE + x] = reg[i][e];
     }
@@ -218,7 +232,7 @@ struct FastLoader {
         const int k = v / (BX / VW), xv = v % (BX / VW);
         ptr[i] = base + (x0 + xv * VW) + (int64_t)(k0 + k) * ld;
       } else {
-        const int x = v / (BK / VW), kv = v % (BK / VW);
+        const int x = kcontig_x<BK / VW>(v), kv = kcontig_kv<BK / VW>(v);
         ptr[i] = base + (k0 + kv * VW) + (int64_t)(x0 + x) * ld;
       }
     }
