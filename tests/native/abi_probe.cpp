@@ -1,6 +1,8 @@
 // Stand-alone caller of the C ABI: no Python, no torch, only the HIP runtime for device memory.
 //
 //   abi_probe [rows cols [repeats [copies]]]
+//   abi_probe qr n          QR of a pseudo-random n x n matrix (library-owned workspace), Q checked on the host
+//   abi_probe eigh n        fp64 eigendecomposition of a symmetric n x n matrix, checked on the host
 //
 // 1. `copies` layout copies of a rows x cols fp32 matrix (4*rows*cols bytes read, as many written):
 //    the kernel of known size that hardware-counter readings of a profiled run are scaled by.
@@ -15,6 +17,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <string>
 #include <vector>
 
 #include "soap_mi355.h"
@@ -46,7 +49,78 @@ static float host_value(uint64_t index) {
   return (float)((double)(x & 0xFFFFFF) / (double)0x1000000 - 0.5);
 }
 
+// Q^T Q = I and Q^T A upper triangular for soapmi_qr_f32 with a NULL workspace.
+static int check_qr(int64_t n) {
+  std::vector<float> a((size_t)n * n), q((size_t)n * n);
+  for (size_t i = 0; i < a.size(); ++i) a[i] = host_value(i + 17);
+  float *d_a, *d_q;
+  HIP_OK(hipMalloc((void**)&d_a, a.size() * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_q, q.size() * sizeof(float)));
+  HIP_OK(hipMemcpy(d_a, a.data(), a.size() * sizeof(float), hipMemcpyHostToDevice));
+  ABI_OK(soapmi_qr_f32(d_a, d_q, n, n, n, nullptr, 0, nullptr));
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(q.data(), d_q, q.size() * sizeof(float), hipMemcpyDeviceToHost));
+  double worst_orth = 0.0, worst_lower = 0.0;
+  for (int64_t i = 0; i < n; ++i)
+    for (int64_t j = 0; j < n; ++j) {
+      double dot = 0.0, r = 0.0;
+      for (int64_t k = 0; k < n; ++k) {
+        dot += (double)q[k + i * n] * q[k + j * n];
+        r += (double)q[k + i * n] * a[k + j * n];  // R[i, j] = (Q^T A)[i, j]
+      }
+      worst_orth = std::fmax(worst_orth, std::fabs(dot - (i == j ? 1.0 : 0.0)));
+      if (i > j) worst_lower = std::fmax(worst_lower, std::fabs(r));
+    }
+  std::printf("qr n=%lld: max |Q^T Q - I| %.3e, max |strictly lower (Q^T A)| %.3e\n", (long long)n, worst_orth,
+              worst_lower);
+  hipFree(d_a); hipFree(d_q);
+  if (!(worst_orth < 1e-4 && worst_lower < 1e-4 * std::sqrt((double)n))) return 4;
+  std::printf("ok\n");
+  return 0;
+}
+
+// A Z = Z diag(w), Z^T Z = I, w ascending for soapmi_eigh_f64 with a NULL workspace.
+static int check_eigh(int64_t n) {
+  std::vector<double> a((size_t)n * n), z((size_t)n * n), w((size_t)n);
+  for (int64_t i = 0; i < n; ++i)
+    for (int64_t j = 0; j <= i; ++j) a[i + j * n] = a[j + i * n] = host_value((uint64_t)(i * n + j) + 5);
+  double *d_a, *d_z, *d_w;
+  HIP_OK(hipMalloc((void**)&d_a, a.size() * sizeof(double)));
+  HIP_OK(hipMalloc((void**)&d_z, z.size() * sizeof(double)));
+  HIP_OK(hipMalloc((void**)&d_w, w.size() * sizeof(double)));
+  HIP_OK(hipMemcpy(d_a, a.data(), a.size() * sizeof(double), hipMemcpyHostToDevice));
+  ABI_OK(soapmi_eigh_f64(d_a, d_w, d_z, n, n, n, nullptr, 0, nullptr));
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(z.data(), d_z, z.size() * sizeof(double), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(w.data(), d_w, w.size() * sizeof(double), hipMemcpyDeviceToHost));
+  double worst_res = 0.0, worst_orth = 0.0, scale = 0.0;
+  bool ascending = true;
+  for (int64_t j = 0; j < n; ++j) {
+    scale = std::fmax(scale, std::fabs(w[j]));
+    if (j > 0 && w[j] < w[j - 1]) ascending = false;
+  }
+  for (int64_t j = 0; j < n; ++j) {
+    for (int64_t i = 0; i < n; ++i) {
+      double az = 0.0, dot = 0.0;
+      for (int64_t k = 0; k < n; ++k) {
+        az += a[i + k * n] * z[k + j * n];
+        dot += z[k + i * n] * z[k + j * n];
+      }
+      worst_res = std::fmax(worst_res, std::fabs(az - w[j] * z[i + j * n]));
+      worst_orth = std::fmax(worst_orth, std::fabs(dot - (i == j ? 1.0 : 0.0)));
+    }
+  }
+  std::printf("eigh n=%lld: max |A Z - Z w| / max|w| %.3e, max |Z^T Z - I| %.3e, ascending %d\n", (long long)n,
+              worst_res / scale, worst_orth, (int)ascending);
+  hipFree(d_a); hipFree(d_z); hipFree(d_w);
+  if (!(ascending && worst_res / scale < 1e-12 && worst_orth < 1e-12)) return 4;
+  std::printf("ok\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
+  if (argc == 3 && std::string(argv[1]) == "qr") return check_qr(std::atoll(argv[2]));
+  if (argc == 3 && std::string(argv[1]) == "eigh") return check_eigh(std::atoll(argv[2]));
   const int64_t rows = argc > 2 ? std::atoll(argv[1]) : 4096;
   const int64_t cols = argc > 2 ? std::atoll(argv[2]) : 11008;
   const int repeats = argc > 3 ? std::atoi(argv[3]) : 5;

@@ -16,3 +16,13 @@ def test_rotate_adam_rotate_from_cpp(rows, cols):
                                timeout=100)
     assert completed.returncode == 0, completed.stdout + completed.stderr
     assert completed.stdout.strip().endswith("ok"), completed.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode,size", [("qr", 300), ("eigh", 300)])
+def test_factorisations_from_cpp_with_library_owned_workspace(mode, size):
+    if not PROBE.exists():
+        pytest.fail(f"{PROBE} is not built: run python -m soap_tp_amd.build")
+    completed = subprocess.run([str(PROBE), mode, str(size)], capture_output=True, text=True, timeout=100)
+    assert completed.returncode == 0, completed.stdout + completed.stderr
+    assert completed.stdout.strip().endswith("ok"), completed.stdout
