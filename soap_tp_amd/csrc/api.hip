@@ -34,6 +34,8 @@ static InternalScratch g_scratch[64];
 static std::atomic<int> g_qr_persistent_max_wg{kQrPersistentMaxWg};
 // polls a workgroup spends waiting for another one's message before it gives up (see soapmi_set_option)
 static std::atomic<unsigned> g_message_spin_limit{kQrSpinLimit};
+// panel columns the QR factors per message round (see soapmi_set_option)
+static std::atomic<int> g_qr_columns_per_round{2};
 static std::mutex g_scratch_mutex;
 
 static int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out) {
@@ -155,6 +157,11 @@ int soapmi_set_option(const char* name, int64_t value) {
     SOAPMI_REQUIRE(value >= 0 && value <= kQrPersistentMaxWg, "qr_persistent_max_workgroups must be in 0..%d",
                    kQrPersistentMaxWg);
     g_qr_persistent_max_wg.store((int)value);
+    return kOk;
+  }
+  if (strcmp(name, "qr_columns_per_round") == 0) {
+    SOAPMI_REQUIRE(value == 1 || value == 2, "qr_columns_per_round must be 1 or 2");
+    g_qr_columns_per_round.store((int)value);
     return kOk;
   }
   if (strcmp(name, "message_spin_limit") == 0) {
@@ -505,7 +512,8 @@ int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t 
   QrWorkspace<float> qws;
   qr_workspace_layout<float>(w, n, &qws);
   return qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws,
-                                     g_qr_persistent_max_wg.load(), g_message_spin_limit.load());
+                                     g_qr_persistent_max_wg.load(), g_message_spin_limit.load(),
+                                     g_qr_columns_per_round.load());
 }
 
 size_t soapmi_power_iteration_qr_workspace_bytes(int64_t n) {

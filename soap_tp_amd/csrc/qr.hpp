@@ -196,10 +196,10 @@ __global__ __launch_bounds__(256) void qr_panel_step_kernel(T* __restrict__ A, i
 // value travels as one 64-bit word {float bits, sequence number} written and read with single-copy
 // atomic accesses, so a reader that sees the expected sequence number has the value with it.  No
 // separate flag, counter or fence is needed, and a column costs one trip through memory.
-// Sequence numbers grow by one per column over the whole factorisation (the host passes the
-// launch's starting value and clears the mailboxes before the first panel), mailboxes alternate
-// between two sets by column parity: a workgroup writes column c+2 only after it has read every
-// workgroup's column c+1, which those wrote after they had read column c.
+// Sequence numbers grow by one per message round over the whole factorisation (the host passes
+// the launch's starting value and clears the mailboxes before the first panel), mailboxes
+// alternate between two sets by round parity: a workgroup writes round t+2 only after it has read
+// every workgroup's round t+1, which those wrote after they had read round t.
 // Besides A the kernel writes the panel's reflectors in clean form (unit diagonal, zeros above) to
 // vout, the operand of the block-reflector products.
 // Requirements: all workgroups of the launch are resident at the same time (the host launches at
@@ -213,8 +213,8 @@ __device__ __forceinline__ unsigned long long mailbox_pack(float value, unsigned
   return ((unsigned long long)seq << 32) | (unsigned long long)__float_as_uint(value);
 }
 
-// Reads `count` (<= 8) mailbox words until all carry `seq`; false after too many polls or once the
-// error flag is up.
+// Reads COUNT mailbox words until all carry `seq`; false after too many polls or once the error
+// flag is up.
 template <int COUNT>
 __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&slot)[COUNT], const bool (&used)[COUNT],
                                              unsigned seq, const int* error, unsigned spin_limit,
@@ -241,27 +241,68 @@ __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&s
   }
 }
 
+// Householder scalars of a column with leading entry alpha and squared norm x2 of the rest.
+// A column whose squared norm is at most `floor2` is left alone (tau = 0): see kQrNegligible.
+struct Reflector {
+  float beta, tau, scale;
+};
+__device__ __forceinline__ Reflector make_reflector(float alpha, float x2, float floor2) {
+  Reflector h{alpha, 0.0f, 0.0f};
+  if (x2 > 0.0f && alpha * alpha + x2 > floor2) {
+    const float nrm = sqrtf(alpha * alpha + x2);
+    h.beta = (alpha >= 0.0f) ? -nrm : nrm;
+    h.tau = (h.beta - alpha) / h.beta;
+    h.scale = 1.0f / (alpha - h.beta);
+  }
+  return h;
+}
+
+// A column whose squared norm has fallen below kQrNegligible times the largest one met so far in
+// its panel (a norm ratio of 1e-12) gets no reflector.  Such columns are rounding residue of
+// exactly dependent columns; left to themselves they shrink by 1e-7 per column until their
+// squares underflow, and a reflector built from underflowed sums is not orthogonal (LAPACK's
+// slarfg rescales instead, which a norm that comes out of a reduction cannot do in place).
+// What stays below the diagonal of R is below 1e-12 of the panel's scale; Q stays orthogonal.
+constexpr float kQrNegligible = 1e-24f;
+
+// Two columns per message round.  Besides the dot products of column j with the remaining columns
+// (over the rows below the pivot) a round also reduces those of column j+1 as it stands (over the
+// rows below ITS pivot) and broadcasts both pivot rows.  Once reflector j is known, what column
+// j+1 and its dot products become after applying it follows by a rank-one correction,
+//   a'_k = a_k - tc_k v,  <a'_1, a'_k> = <a_1, a_k> - tc_k s <a_0, a_1> - tc_1 s <a_0, a_k> + tc_1 tc_k s^2 <a_0, a_0>
+// (s = reflector j's scale, sums over the rows below pivot j+1), so reflector j+1 needs no second
+// round.  The corrected squared norm of column j+1 is a difference: when it comes out below
+// kQrPairGuard times the size of the terms it is formed from (column j+1 nearly parallel to
+// column j, cancellation), the pair is abandoned, only reflector j is applied, and column j+1 gets a round of its own with
+// directly computed sums.  Every workgroup takes that decision from the same numbers.
+constexpr float kQrPairGuard = 0.25f;
+
 __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restrict__ A, int64_t lda, int n, int p,
                                                                   int pe, unsigned long long* part,
                                                                   unsigned long long* piv, float* __restrict__ tau,
                                                                   unsigned seq_base, int* error, int nwg,
                                                                   unsigned spin_limit, float* __restrict__ vout,
-                                                                  int64_t ldv, int vrow0) {
+                                                                  int64_t ldv, int vrow0, int pairs) {
   using T = float;
   constexpr int NB = kQrNb;
-  __shared__ T s_tc[NB];
-  __shared__ T s_wave[4][NB];
-  __shared__ T s_sum8[8][NB];
-  __shared__ T s_piv_out[NB];
-  __shared__ T s_piv[NB];
-  __shared__ T s_scal[3];
+  __shared__ T s_wave[4][2 * NB];
+  __shared__ T s_sum4[4][2 * NB];
+  __shared__ T s_piv_out[2 * NB];
+  __shared__ T s_tot[2 * NB];   // [0, NB): column j's sums, [NB, 2 NB): column j+1's
+  __shared__ T s_piv[2 * NB];   // pivot rows j and j+1
+  __shared__ T s_tc[2][NB];
+  __shared__ T s_scal[8];
+  __shared__ int s_pair_ok;
   __shared__ int s_fail;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wg = blockIdx.x;
   const int r = p + wg * 256 + tid;
   const int nbw = pe - p;
   const bool live = r < n;
-  if (tid == 0) s_fail = 0;
+  if (tid == 0) {
+    s_fail = 0;
+    s_scal[6] = T(0);
+  }
   // vout (rows vrow0.., one column per panel column) receives the reflectors in clean form: zeros
   // above the unit diagonal, including the vrow0 - p ... rows above the panel that no thread owns
   if (wg == 0) {
@@ -272,13 +313,15 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
 #pragma unroll
   for (int c = 0; c < NB; ++c) a[c] = (live && c < nbw) ? A[r + (int64_t)(p + c) * lda] : T(0);
 
-  for (int c = 0; c < nbw; ++c) {
+  int c = 0;
+  for (unsigned round = 0; c < nbw; ++round) {
     const int j = p + c;
-    const unsigned seq = seq_base + (unsigned)c + 1u;
-    unsigned long long* part_c = part + (size_t)(c & 1) * kQrPersistentMaxWg * NB;
-    unsigned long long* piv_c = piv + (c & 1) * NB;
-    const bool owns_pivot = j >= p + wg * 256 && j < p + wg * 256 + 256;
-    // dot products of column j with the remaining panel columns over the rows below the pivot
+    const bool pair = pairs != 0 && c + 1 < nbw;
+    const int width = pair ? 2 * NB : NB;  // values per workgroup in this round
+    const unsigned seq = seq_base + round + 1u;
+    unsigned long long* part_c = part + (size_t)(round & 1) * kQrPersistentMaxWg * 2 * NB;
+    unsigned long long* piv_c = piv + (round & 1) * 2 * NB;
+    // dot products over the rows below the pivot(s)
     {
       const bool below = live && r > j;
       T vals[NB];
@@ -291,33 +334,49 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
         for (int k = 0; k < NB; ++k) s_piv_out[k] = a[k];
       }
     }
+    if (pair) {
+      const bool below = live && r > j + 1;
+      T vals[NB];
+#pragma unroll
+      for (int k = 0; k < NB; ++k) vals[k] = below ? a[1] * a[k] : T(0);
+      const T total = wave_reduce_32<T>(vals, lane);
+      if ((lane & 1) == 0) s_wave[wave][NB + ((lane >> 1) & 31)] = total;
+      if (live && r == j + 1) {
+#pragma unroll
+        for (int k = 0; k < NB; ++k) s_piv_out[NB + k] = a[k];
+      }
+    }
     __syncthreads();
-    if (tid < NB) {
+    if (tid < width) {
       const T sum = (s_wave[0][tid] + s_wave[1][tid]) + (s_wave[2][tid] + s_wave[3][tid]);
-      __hip_atomic_store(part_c + wg * NB + tid, mailbox_pack(sum, seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (owns_pivot)
+      __hip_atomic_store(part_c + wg * 2 * NB + tid, mailbox_pack(sum, seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int pivot_row = tid < NB ? j : j + 1;
+      if (pivot_row >= p + wg * 256 && pivot_row < p + wg * 256 + 256)  // this workgroup owns that pivot row
         __hip_atomic_store(piv_c + tid, mailbox_pack(s_piv_out[tid], seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     {
-      // fixed-order sum of the per-workgroup partials, as in qr_panel_step_kernel
-      const int k = tid & (NB - 1), g = tid >> 5;
+      // fixed-order sums of the per-workgroup partials: thread (k, g) takes value k of the workgroups
+      // g, g + 4, ..., sixteen loads in flight
+      const int k = tid & (2 * NB - 1), g = tid >> 6;
       T s = T(0);
       bool ok = true;
-      for (int w0 = g; w0 < nwg && ok; w0 += 64) {
-        const unsigned long long* slot[8];
-        bool used[8];
-        float v[8];
+      if (k < width) {
+        for (int w0 = g; w0 < nwg && ok; w0 += 64) {
+          const unsigned long long* slot[16];
+          bool used[16];
+          float v[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          used[u] = w0 + 8 * u < nwg;
-          slot[u] = part_c + (used[u] ? (w0 + 8 * u) : 0) * NB + k;
+          for (int u = 0; u < 16; ++u) {
+            used[u] = w0 + 4 * u < nwg;
+            slot[u] = part_c + (used[u] ? (w0 + 4 * u) : 0) * 2 * NB + k;
+          }
+          ok = mailbox_wait<16>(slot, used, seq, error, spin_limit, v);
+#pragma unroll
+          for (int u = 0; u < 16; ++u) s += v[u];
         }
-        ok = mailbox_wait<8>(slot, used, seq, error, spin_limit, v);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
       }
-      s_sum8[g][k] = s;
-      if (tid < NB && ok) {
+      s_sum4[g][k] = s;
+      if (tid < width && ok) {
         const unsigned long long* slot[1] = {piv_c + tid};
         const bool used[1] = {true};
         float v[1];
@@ -331,51 +390,107 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
     }
     __syncthreads();
     if (s_fail) return;
+    if (tid < width) s_tot[tid] = (s_sum4[0][tid] + s_sum4[1][tid]) + (s_sum4[2][tid] + s_sum4[3][tid]);
+    __syncthreads();
     if (tid < NB) {
-      T x2 = T(0), dot = T(0);
-#pragma unroll
-      for (int g = 0; g < 8; ++g) {
-        x2 += s_sum8[g][0];
-        dot += s_sum8[g][tid];
+      const int k = tid;
+      const T seen = s_scal[6];  // largest squared column norm of this panel so far (0 at its first column)
+      const Reflector h0 = make_reflector(s_piv[0], s_tot[0], kQrNegligible * seen);
+      T seen_next = fmaxf(seen, s_piv[0] * s_piv[0] + s_tot[0]);
+      const T tc0 = (k >= 1) ? h0.tau * (s_piv[k] + h0.scale * s_tot[k]) : T(0);
+      s_tc[0][k] = tc0;
+      if (k == 0) {
+        s_scal[0] = h0.scale; s_scal[1] = h0.beta; s_scal[2] = h0.tau;
       }
-      const T alpha = s_piv[0];
-      T beta = alpha, tauv = T(0), scale = T(0);
-      if (x2 > T(0)) {
-        const T nrm = sqrt(alpha * alpha + x2);
-        beta = (alpha >= T(0)) ? -nrm : nrm;
-        tauv = (beta - alpha) / beta;
-        scale = T(1) / (alpha - beta);
+      T seen_out = seen_next;
+      if (pair) {
+        // row j+1 and the sums over the rows below it, after reflector j
+        const T q0 = s_piv[NB];                              // a_0[j+1]
+        const T v0_next = h0.scale * q0;                     // v[j+1]
+        const T tc0_1 = h0.tau * (s_piv[1] + h0.scale * s_tot[1]);
+        const T piv1 = s_piv[NB + k] - tc0 * v0_next;        // a'_k[j+1], k >= 1
+        const T sp_k = s_tot[k] - q0 * s_piv[NB + k];        // <a_0, a_k> below row j+1
+        const T sp_0 = s_tot[0] - q0 * q0;
+        const T sp_1 = s_tot[1] - q0 * s_piv[NB + 1];
+        const T u_k = s_tot[NB + k] - tc0 * h0.scale * sp_1 - tc0_1 * h0.scale * sp_k +
+                      tc0_1 * tc0 * h0.scale * h0.scale * sp_0;
+        // lane 1 holds the corrected squared norm of column j+1 below its pivot and its pivot entry
+        // (the last column of the matrix has nothing below its pivot: exactly zero, so tau = 0 as in LAPACK)
+        const T x2_1 = (j + 1 < n - 1) ? __shfl(u_k, 1, 64) : T(0), alpha1 = __shfl(piv1, 1, 64);
+        // size of the terms the corrected norm is the difference of (all three are >= 0 in exact arithmetic)
+        const T magnitude = s_tot[NB + 1] + T(2) * fabsf(tc0_1 * h0.scale * sp_1) +
+                            tc0_1 * tc0_1 * h0.scale * h0.scale * fabsf(sp_0);
+        const bool ok = (x2_1 - x2_1 == T(0)) && x2_1 >= kQrPairGuard * magnitude;  // finite and no cancellation
+        const Reflector h1 = make_reflector(alpha1, fmaxf(x2_1, T(0)), kQrNegligible * seen_next);
+        if (ok) seen_next = fmaxf(seen_next, alpha1 * alpha1 + fmaxf(x2_1, T(0)));
+        s_tc[1][k] = (k >= 2) ? h1.tau * (piv1 + h1.scale * u_k) : T(0);
+        seen_out = seen_next;
+        if (k == 0) {
+          s_scal[3] = h1.scale; s_scal[4] = h1.beta; s_scal[5] = h1.tau;
+          s_pair_ok = ok ? 1 : 0;
+        }
+      } else if (k == 0) {
+        s_pair_ok = 0;
       }
-      s_tc[tid] = (tid >= 1) ? tauv * (s_piv[tid] + scale * dot) : T(0);
-      if (tid == 0) {
-        s_scal[0] = scale; s_scal[1] = beta; s_scal[2] = tauv;
-      }
+      // every lane read s_scal[6] above; lane 0 of the same wavefront may now replace it
+      if (k == 0) s_scal[6] = seen_out;
     }
     __syncthreads();
-    const T scale = s_scal[0], beta = s_scal[1], tauv = s_scal[2];
-    if (live && r >= j) {
-      if (r > j) {
-        const T v = a[0] * scale;
-        a[0] = v;
+    const bool two = s_pair_ok != 0;
+    {
+      const T scale = s_scal[0], beta = s_scal[1], tauv = s_scal[2];
+      if (live && r >= j) {
+        if (r > j) {
+          const T v = a[0] * scale;
+          a[0] = v;
 #pragma unroll
-        for (int k = 1; k < NB; ++k) a[k] -= s_tc[k] * v;
-      } else {
-        a[0] = beta;
+          for (int k = 1; k < NB; ++k) a[k] -= s_tc[0][k] * v;
+        } else {
+          a[0] = beta;
 #pragma unroll
-        for (int k = 1; k < NB; ++k) a[k] -= s_tc[k];
-        tau[j] = tauv;
+          for (int k = 1; k < NB; ++k) a[k] -= s_tc[0][k];
+          tau[j] = tauv;
+        }
+      }
+      if (live) {
+        A[r + (int64_t)j * lda] = a[0];  // column j is final
+        vout[(r - vrow0) + (int64_t)c * ldv] = (r > j) ? a[0] : (r == j ? T(1) : T(0));
       }
     }
-    if (live) {
-      A[r + (int64_t)j * lda] = a[0];  // column j is final
-      vout[(r - vrow0) + (int64_t)c * ldv] = (r > j) ? a[0] : (r == j ? T(1) : T(0));
-    }
+    if (two) {
+      const T scale = s_scal[3], beta = s_scal[4], tauv = s_scal[5];
+      const int j1 = j + 1;
+      if (live && r >= j1) {
+        if (r > j1) {
+          const T v = a[1] * scale;
+          a[1] = v;
 #pragma unroll
-    for (int k = 0; k + 1 < NB; ++k) a[k] = a[k + 1];
-    a[NB - 1] = T(0);
-    // No barrier here: the shared arrays of the next column's first phase (s_wave, s_piv_out) were
-    // last read before the barrier that follows the mailbox phase, and s_tc / s_scal are rewritten
-    // only behind the next such barrier, which every wavefront reaches after this point.
+          for (int k = 2; k < NB; ++k) a[k] -= s_tc[1][k] * v;
+        } else {
+          a[1] = beta;
+#pragma unroll
+          for (int k = 2; k < NB; ++k) a[k] -= s_tc[1][k];
+          tau[j1] = tauv;
+        }
+      }
+      if (live) {
+        A[r + (int64_t)j1 * lda] = a[1];
+        vout[(r - vrow0) + (int64_t)(c + 1) * ldv] = (r > j1) ? a[1] : (r == j1 ? T(1) : T(0));
+      }
+#pragma unroll
+      for (int k = 0; k + 2 < NB; ++k) a[k] = a[k + 2];
+      a[NB - 2] = T(0);
+      a[NB - 1] = T(0);
+      c += 2;
+    } else {
+#pragma unroll
+      for (int k = 0; k + 1 < NB; ++k) a[k] = a[k + 1];
+      a[NB - 1] = T(0);
+      c += 1;
+    }
+    // No barrier here: the shared arrays of the next round's first phase (s_wave, s_piv_out) were
+    // last read before the barrier that follows the mailbox phase, and the arrays read above are
+    // rewritten only behind the next such barrier, which every wavefront reaches after this point.
   }
 }
 
@@ -669,8 +784,8 @@ struct QrWorkspace {
   T* tau;     // n
   T* part;    // 2 x nwg x NB   partials of the launch-per-column fallback
   T* piv;     // 2 x NB
-  unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x NB   mailboxes of the persistent panel kernel
-  unsigned long long* mail_piv;   // 2 x NB
+  unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x 2 NB   mailboxes of the persistent panel kernel
+  unsigned long long* mail_piv;   // 2 x 2 NB
   unsigned* sync;  // [1] error flag of the persistent panel kernel
 };
 
@@ -684,8 +799,8 @@ static inline void qr_workspace_layout(WS& ws, int64_t n, QrWorkspace<T>* out) {
   q.tau = ws.template take<T>((size_t)n);
   q.part = ws.template take<T>((size_t)2 * nwg * kQrNb);
   q.piv = ws.template take<T>(2 * kQrNb);
-  q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * kQrNb);
-  q.mail_piv = ws.template take<unsigned long long>(2 * kQrNb);
+  q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * 2 * kQrNb);
+  q.mail_piv = ws.template take<unsigned long long>(2 * 2 * kQrNb);
   q.sync = ws.template take<unsigned>(64);
   if (out) *out = q;
 }
@@ -704,7 +819,7 @@ static inline size_t qr_workspace_bytes(int64_t n) {
 template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
                                        const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
-                                       unsigned spin_limit = kQrSpinLimit) {
+                                       unsigned spin_limit = kQrSpinLimit, int columns_per_round = 2) {
   const int NB = kQrNb, OB = kBrMax;
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
@@ -714,7 +829,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
   hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
   {
     // mail_part and mail_piv are adjacent: one clear covers both (sequence number 0 = "nothing yet")
-    const int words = 2 * (2 * kQrPersistentMaxWg * kQrNb + 2 * kQrNb);
+    const int words = 2 * (2 * kQrPersistentMaxWg * 2 * kQrNb + 2 * 2 * kQrNb);
     hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3((words + 255) / 256), dim3(256), 0, s,
                        reinterpret_cast<unsigned*>(ws.mail_part), words);
   }
@@ -737,7 +852,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
                            ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
-                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P);
+                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, columns_per_round >= 2 ? 1 : 0);
         seq_base += (unsigned)nbw;
       } else {
         for (int j = p - 1; j < pe; ++j) {
