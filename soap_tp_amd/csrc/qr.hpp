@@ -678,11 +678,11 @@ static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws
 }
 
 // Number of K slices for a tall-skinny product with `tiles` output tiles, K = rows, an M x N
-// output: enough slices to occupy the chip (about 512 workgroups), at least 256 rows each, and no
+// output: enough slices to occupy the chip (about 512 workgroups), at least 128 rows each, and no
 // more partial results than the split-K buffer (kBrSplits * kBrMax * ldv elements) holds.
 static inline int split_count(int64_t tiles, int rows, int M, int N, int64_t ldv) {
-  if (rows < 1024) return 1;
-  int64_t splits = std::min<int64_t>(ceil_div64(512, tiles), rows / 256);
+  if (rows < 512) return 1;
+  int64_t splits = std::min<int64_t>(ceil_div64(512, tiles), rows / 128);
   const int64_t capacity = (int64_t)kBrSplits * kBrMax * ldv / std::max<int64_t>(1, (int64_t)M * N);
   splits = std::min<int64_t>(splits, std::min<int64_t>(capacity, 64));
   return (int)std::max<int64_t>(splits, 1);
