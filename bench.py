@@ -214,6 +214,8 @@ def run_layer(device, steps=30, rank=64):
     end.record()
     torch.cuda.synchronize()
     total_ms = begin.elapsed_time(end)
+    if not all(bool(torch.isfinite(parameter).all()) for parameter in parameters):
+        raise RuntimeError("a parameter of the layer run is not finite")
     flops = sum(5.0 * m * n * (m + n) for m, n in shapes)
     return {"workload": "4 x 4096x4096, 2 x 4096x14336, 1 x 14336x4096, rank 64, refresh every 10, "
                         "optimizer wrapper with 2 side streams", "steps": steps,
