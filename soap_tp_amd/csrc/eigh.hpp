@@ -64,7 +64,7 @@ static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, i
   if (rc) return rc;
   rc = stedc<T>(s, n, ws.d, ws.e, w, Z, ldz, ws.dc);
   if (rc) return rc;
-  // Z <- H_0 H_1 ... H_{n-2} Z, 128-wide block reflectors applied last block first.
+  // Z <- H_0 H_1 ... H_{n-2} Z, kBrMax-wide block reflectors applied last block first.
   const int nref = n - 1;  // reflector j lives in column j, rows j+1..n-1
   if (nref <= 0) return kOk;  // n == 1: no column kernel ran
   constexpr int OB = kBrMax;

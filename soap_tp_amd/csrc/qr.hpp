@@ -2,11 +2,14 @@
 // power-iteration refresh of a SOAP eigenbasis (what the reference obtains from SLATE's
 // geqrf + unmqr on the identity: src/soap_tp/csrc/slate_bindings.cpp:176-185).
 //
-// Panel (NB = 32 columns): one launch per column.  A workgroup owns 256 rows, one per thread,
-// and keeps its row of the panel in registers.  Launch j applies reflector j (whose dot
-// products with the remaining panel columns were reduced by launch j-1) and, in the same pass,
-// reduces the dot products reflector j+1 needs: a 32-value butterfly over the wavefront, then
-// a fixed-order sum over workgroups.  No atomics, so results do not depend on scheduling.
+// Panel (NB = 32 columns): a workgroup owns 256 rows, one per thread, and keeps its row of the
+// panel in registers.  Normally the whole panel runs in one persistent launch whose workgroups
+// exchange partial dot products through device memory, two columns per exchange
+// (qr_panel_persistent_kernel); beyond kQrPersistentMaxWg workgroups it runs one launch per column
+// (qr_panel_step_kernel: launch j applies reflector j, whose dot products with the remaining
+// panel columns were reduced by launch j-1, and in the same pass reduces the dot products reflector
+// j+1 needs).  Reductions are a 32-value butterfly over the wavefront, then a fixed-order sum over
+// workgroups: no atomics on data, so results do not depend on scheduling.
 // Trailing matrix and Q formation: compact-WY block reflectors on the MFMA GEMM.
 #pragma once
 #include <type_traits>
@@ -814,8 +817,8 @@ static inline size_t qr_workspace_bytes(int64_t n) {
 
 // geqrf in place on A (n x n), then the explicit Q into Qout (n x n).  A is destroyed.
 // Two levels of blocking: 32-column panels (register-resident column steps) are applied only
-// inside their 128-column outer block; the trailing matrix and Q see 128-wide block reflectors,
-// whose products have K = 128 and run on the full-size MFMA tile.
+// inside their kBrMax-column outer block; the trailing matrix and Q see kBrMax-wide block
+// reflectors, whose products have K = kBrMax and run on the full-size MFMA tile.
 template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
                                        const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
