@@ -11,8 +11,9 @@
 //
 // Per merge: sort the eigenvalues of the two children (bitonic, batched); deflate (one
 // sequential scan, staged through LDS); apply the deflation rotations and gather the surviving
-// eigenvector columns; solve the secular equation, one thread per root, with a bracketed
-// rational ("middle way") iteration that falls back to bisection; recompute the update vector
+// eigenvector columns; solve the secular equation with a bracketed rational ("middle way")
+// iteration that falls back to bisection, one thread per root in small merges and one wavefront
+// per root (poles spread over the lanes) in merges of 256 and more; recompute the update vector
 // from the roots; form the k x k eigenvector matrix of the rank-one update; multiply (MFMA).
 // Eigenvector columns are not kept in sorted order between levels (the sort permutation is
 // recomputed where it is needed); one final sort orders the result.
