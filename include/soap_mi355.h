@@ -49,11 +49,11 @@ const char* soapmi_last_error(void);
  *   "qr_persistent_max_workgroups"  0..128 (default 128): a QR panel whose grid (rows / 256) fits
  *       runs as one persistent launch whose workgroups exchange partial sums through device memory;
  *       larger panels, or all panels with 0, run one launch per column instead.
- *   "qr_columns_per_round"  1 or 2 (default 2): panel columns the persistent QR panel kernel factors per
- *       exchange of partial sums.  With 2 the second column's reflector follows from the first
- *       one's by a rank-one correction of dot products taken in the same exchange (guarded: a pair
- *       whose corrected norm shows cancellation falls back to one column); 1 computes every
- *       column's sums directly.
+ *   "qr_columns_per_round"  1..4 (default 4): panel columns the persistent QR panel kernel factors per
+ *       exchange of partial sums.  The exchange carries the dot products of all the round's columns;
+ *       the reflectors after the first follow from those by rank-one corrections (guarded: a
+ *       column whose corrected norm shows cancellation ends the round and starts the next one with
+ *       directly computed sums); 1 computes every column's sums directly.
  *   "message_spin_limit"  0..4194304 (default 4194304): how many times a workgroup of the QR panel
  *       kernel or of the tridiagonalisation's column kernel polls for another workgroup's message
  *       before it gives up.  Giving up never hangs and never passes silently: the kernels leave,

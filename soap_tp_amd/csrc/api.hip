@@ -35,7 +35,7 @@ static std::atomic<int> g_qr_persistent_max_wg{kQrPersistentMaxWg};
 // polls a workgroup spends waiting for another one's message before it gives up (see soapmi_set_option)
 static std::atomic<unsigned> g_message_spin_limit{kQrSpinLimit};
 // panel columns the QR factors per message round (see soapmi_set_option)
-static std::atomic<int> g_qr_columns_per_round{2};
+static std::atomic<int> g_qr_columns_per_round{kQrRoundMax};
 static std::mutex g_scratch_mutex;
 
 static int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out) {
@@ -160,7 +160,7 @@ int soapmi_set_option(const char* name, int64_t value) {
     return kOk;
   }
   if (strcmp(name, "qr_columns_per_round") == 0) {
-    SOAPMI_REQUIRE(value == 1 || value == 2, "qr_columns_per_round must be 1 or 2");
+    SOAPMI_REQUIRE(value >= 1 && value <= kQrRoundMax, "qr_columns_per_round must be in 1..%d", kQrRoundMax);
     g_qr_columns_per_round.store((int)value);
     return kOk;
   }

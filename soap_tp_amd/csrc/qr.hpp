@@ -74,16 +74,45 @@ __device__ __forceinline__ void butterfly_stage_swap(T (&vals)[32]) {
   for (int c = 0; c < HALF; ++c) vals[c] = swap_add<WIDE32>(vals[c], vals[c + HALF]);
 }
 
+// The narrow stages on data-parallel-primitive moves (no trip through the LDS crossbar): the
+// partner is lane ^ 15 (row_mirror), lane ^ 7 (row_half_mirror), lane ^ 2 and lane ^ 1 (quad_perm).
+// Together with the two swap stages (lane ^ 32, lane ^ 16) these six masks reach every lane of the
+// wavefront, and which half a lane keeps at a stage is decided by one bit of its own number, so the
+// value index a lane ends up with is the same as with the plain xor pattern.
+template <int CTRL>
+__device__ __forceinline__ float dpp_partner(float v) {
+  return __uint_as_float((unsigned)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_partner(double v) {
+  const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, 0xF, 0xF, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, 0xF, 0xF, false);
+  return __hiloint2double(hi, lo);
+}
+
+constexpr int kDppRowMirror = 0x140, kDppRowHalfMirror = 0x141, kDppQuadXor2 = 0x4E, kDppQuadXor1 = 0xB1;
+
+template <typename T, int HALF, int BIT, int CTRL>
+__device__ __forceinline__ void butterfly_stage_dpp(T (&vals)[32], int lane) {
+  const bool upper = (lane & BIT) != 0;
+#pragma unroll
+  for (int c = 0; c < HALF; ++c) {
+    const T send = upper ? vals[c] : vals[c + HALF];
+    const T keep = upper ? vals[c + HALF] : vals[c];
+    vals[c] = keep + dpp_partner<CTRL>(send);
+  }
+}
+
 // After the call lane l holds, in the return value, the sum over the wavefront of vals[(l>>1)&31].
 // Stages are spelled out so that every register index is a compile-time constant.
 template <typename T>
 __device__ __forceinline__ T wave_reduce_32(T (&vals)[32], int lane) {
   butterfly_stage_swap<T, 16, true>(vals);
   butterfly_stage_swap<T, 8, false>(vals);
-  butterfly_stage<T, 4, 8>(vals, lane);
-  butterfly_stage<T, 2, 4>(vals, lane);
-  butterfly_stage<T, 1, 2>(vals, lane);
-  return vals[0] + __shfl_xor(vals[0], 1, 64);
+  butterfly_stage_dpp<T, 4, 8, kDppRowMirror>(vals, lane);
+  butterfly_stage_dpp<T, 2, 4, kDppRowHalfMirror>(vals, lane);
+  butterfly_stage_dpp<T, 1, 2, kDppQuadXor2>(vals, lane);
+  return vals[0] + dpp_partner<kDppQuadXor1>(vals[0]);
 }
 
 template <typename T>
@@ -268,34 +297,74 @@ __device__ __forceinline__ Reflector make_reflector(float alpha, float x2, float
 // What stays below the diagonal of R is below 1e-12 of the panel's scale; Q stays orthogonal.
 constexpr float kQrNegligible = 1e-24f;
 
-// Two columns per message round.  Besides the dot products of column j with the remaining columns
-// (over the rows below the pivot) a round also reduces those of column j+1 as it stands (over the
-// rows below ITS pivot) and broadcasts both pivot rows.  Once reflector j is known, what column
-// j+1 and its dot products become after applying it follows by a rank-one correction,
-//   a'_k = a_k - tc_k v,  <a'_1, a'_k> = <a_1, a_k> - tc_k s <a_0, a_1> - tc_1 s <a_0, a_k> + tc_1 tc_k s^2 <a_0, a_0>
-// (s = reflector j's scale, sums over the rows below pivot j+1), so reflector j+1 needs no second
-// round.  The corrected squared norm of column j+1 is a difference: when it comes out below
-// kQrPairGuard times the size of the terms it is formed from (column j+1 nearly parallel to
-// column j, cancellation), the pair is abandoned, only reflector j is applied, and column j+1 gets a round of its own with
-// directly computed sums.  Every workgroup takes that decision from the same numbers.
-constexpr float kQrPairGuard = 0.25f;
+// Value of `v` in lane `LANE` (a compile-time constant) as a wavefront-uniform scalar.
+template <int LANE>
+__device__ __forceinline__ float lane_value(float v) {
+  return __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)__float_as_uint(v), LANE));
+}
+template <int LANE>
+__device__ __forceinline__ double lane_value(double v) {
+  const int lo = __builtin_amdgcn_readlane(__double2loint(v), LANE);
+  const int hi = __builtin_amdgcn_readlane(__double2hiint(v), LANE);
+  return __hiloint2double(hi, lo);
+}
+
+// Broadcast from one of the first kQrRoundMax lanes; `t` is a loop counter of a fully unrolled
+// loop, so the switch folds to one v_readlane (a scalar broadcast instead of a trip through the
+// LDS crossbar).
+__device__ __forceinline__ float round_lane_value(float v, int t) {
+  switch (t) {
+    case 0: return lane_value<0>(v);
+    case 1: return lane_value<1>(v);
+    case 2: return lane_value<2>(v);
+    default: return lane_value<3>(v);
+  }
+}
+
+// a[k] <- a[k + D], zeros shifted in at the end; every index is a compile-time constant in range.
+template <int D>
+__device__ __forceinline__ void shift_left(float (&a)[kQrNb]) {
+#pragma unroll
+  for (int k = 0; k + D < kQrNb; ++k) a[k] = a[k + D];
+#pragma unroll
+  for (int k = kQrNb - D; k < kQrNb; ++k) a[k] = 0.0f;
+}
+
+// Several columns per message round.  A round covers the next `cols` <= kQrRoundMax panel columns
+// j .. j+cols-1.  The workgroups exchange (a) the `cols` pivot rows j .. j+cols-1 in full and (b)
+// the dot products G[t][k] = <a_t, a_k> of those columns with all remaining panel columns over the
+// rows BELOW all the round's pivots.  With that, every workgroup runs the `cols` Householder steps
+// on the compressed problem [pivot rows ; Gram of the rest]: the pivot rows are updated
+// explicitly, and the dot products by the rank-one correction that applying reflector t to the
+// hidden rows implies,
+//   a_k <- a_k - tc_k s a_t   =>   G[i][k] <- G[i][k] - tc_k s G[i][t] - tc_i s G[t][k] + tc_i tc_k s^2 G[t][t]
+// (s = the reflector's scale), so no further exchange is needed inside the round.  From the second
+// step on a column's squared norm below its pivot is partly such a corrected number, a difference.
+// Its terms' sizes are tracked alongside; when the norm falls below kQrRoundGuard times that size
+// (cancellation: the column is nearly in the span of the round's earlier columns) the round ends
+// before that step, the accepted reflectors are applied, and the column starts the next round, where
+// its sums are computed directly.  Every workgroup takes these decisions from the same numbers in
+// the same order.
+constexpr int kQrRoundMax = 4;
+constexpr float kQrRoundGuard = 0.25f;
 
 __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restrict__ A, int64_t lda, int n, int p,
                                                                   int pe, unsigned long long* part,
                                                                   unsigned long long* piv, float* __restrict__ tau,
                                                                   unsigned seq_base, int* error, int nwg,
                                                                   unsigned spin_limit, float* __restrict__ vout,
-                                                                  int64_t ldv, int vrow0, int pairs) {
+                                                                  int64_t ldv, int vrow0, int cols_cap) {
   using T = float;
-  constexpr int NB = kQrNb;
-  __shared__ T s_wave[4][2 * NB];
-  __shared__ T s_sum4[4][2 * NB];
-  __shared__ T s_piv_out[2 * NB];
-  __shared__ T s_tot[2 * NB];   // [0, NB): column j's sums, [NB, 2 NB): column j+1's
-  __shared__ T s_piv[2 * NB];   // pivot rows j and j+1
-  __shared__ T s_tc[2][NB];
-  __shared__ T s_scal[8];
-  __shared__ int s_pair_ok;
+  constexpr int NB = kQrNb, S = kQrRoundMax, W = S * NB;  // W values per workgroup and round at most
+  __shared__ T s_wave[4][W];
+  __shared__ T s_sum2[2][W];
+  __shared__ T s_piv_out[W];
+  __shared__ T s_tot[W];    // s_tot[t * NB + k] = G[t][k]
+  __shared__ T s_piv[W];    // s_piv[t * NB + k] = entry k of pivot row j + t
+  __shared__ T s_tc[S][NB];
+  __shared__ T s_scal[S][3];  // scale, beta, tau of the round's reflectors
+  __shared__ T s_seen;        // largest squared column norm of this panel so far
+  __shared__ int s_accepted;
   __shared__ int s_fail;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wg = blockIdx.x;
@@ -304,7 +373,7 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
   const bool live = r < n;
   if (tid == 0) {
     s_fail = 0;
-    s_scal[6] = T(0);
+    s_seen = T(0);
   }
   // vout (rows vrow0.., one column per panel column) receives the reflectors in clean form: zeros
   // above the unit diagonal, including the vrow0 - p ... rows above the panel that no thread owns
@@ -319,66 +388,59 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
   int c = 0;
   for (unsigned round = 0; c < nbw; ++round) {
     const int j = p + c;
-    const bool pair = pairs != 0 && c + 1 < nbw;
-    const int width = pair ? 2 * NB : NB;  // values per workgroup in this round
+    const int cols = min(min(cols_cap, S), nbw - c);
+    const int width = cols * NB;  // values per workgroup in this round
     const unsigned seq = seq_base + round + 1u;
-    unsigned long long* part_c = part + (size_t)(round & 1) * kQrPersistentMaxWg * 2 * NB;
-    unsigned long long* piv_c = piv + (round & 1) * 2 * NB;
-    // dot products over the rows below the pivot(s)
+    unsigned long long* part_c = part + (size_t)(round & 1) * kQrPersistentMaxWg * W;
+    unsigned long long* piv_c = piv + (round & 1) * W;
+    // dot products of the round's columns with all panel columns over the rows below its pivots
     {
-      const bool below = live && r > j;
-      T vals[NB];
+      const bool below = live && r > j + cols - 1;
 #pragma unroll
-      for (int k = 0; k < NB; ++k) vals[k] = below ? a[0] * a[k] : T(0);
-      const T total = wave_reduce_32<T>(vals, lane);
-      if ((lane & 1) == 0) s_wave[wave][(lane >> 1) & 31] = total;
-      if (live && r == j) {
+      for (int t = 0; t < S; ++t) {
+        if (t < cols) {
+          T vals[NB];
 #pragma unroll
-        for (int k = 0; k < NB; ++k) s_piv_out[k] = a[k];
-      }
-    }
-    if (pair) {
-      const bool below = live && r > j + 1;
-      T vals[NB];
+          for (int k = 0; k < NB; ++k) vals[k] = below ? a[t] * a[k] : T(0);
+          const T total = wave_reduce_32<T>(vals, lane);
+          if ((lane & 1) == 0) s_wave[wave][t * NB + ((lane >> 1) & 31)] = total;
+          if (live && r == j + t) {
 #pragma unroll
-      for (int k = 0; k < NB; ++k) vals[k] = below ? a[1] * a[k] : T(0);
-      const T total = wave_reduce_32<T>(vals, lane);
-      if ((lane & 1) == 0) s_wave[wave][NB + ((lane >> 1) & 31)] = total;
-      if (live && r == j + 1) {
-#pragma unroll
-        for (int k = 0; k < NB; ++k) s_piv_out[NB + k] = a[k];
+            for (int k = 0; k < NB; ++k) s_piv_out[t * NB + k] = a[k];
+          }
+        }
       }
     }
     __syncthreads();
     if (tid < width) {
       const T sum = (s_wave[0][tid] + s_wave[1][tid]) + (s_wave[2][tid] + s_wave[3][tid]);
-      __hip_atomic_store(part_c + wg * 2 * NB + tid, mailbox_pack(sum, seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const int pivot_row = tid < NB ? j : j + 1;
+      __hip_atomic_store(part_c + wg * W + tid, mailbox_pack(sum, seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int pivot_row = j + tid / NB;
       if (pivot_row >= p + wg * 256 && pivot_row < p + wg * 256 + 256)  // this workgroup owns that pivot row
         __hip_atomic_store(piv_c + tid, mailbox_pack(s_piv_out[tid], seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     {
       // fixed-order sums of the per-workgroup partials: thread (k, g) takes value k of the workgroups
-      // g, g + 4, ..., sixteen loads in flight
-      const int k = tid & (2 * NB - 1), g = tid >> 6;
+      // g, g + 2, ..., up to thirty-two loads in flight
+      const int k = tid & (W - 1), g = tid >> 7;
       T s = T(0);
       bool ok = true;
       if (k < width) {
         for (int w0 = g; w0 < nwg && ok; w0 += 64) {
-          const unsigned long long* slot[16];
-          bool used[16];
-          float v[16];
+          const unsigned long long* slot[32];
+          bool used[32];
+          float v[32];
 #pragma unroll
-          for (int u = 0; u < 16; ++u) {
-            used[u] = w0 + 4 * u < nwg;
-            slot[u] = part_c + (used[u] ? (w0 + 4 * u) : 0) * 2 * NB + k;
+          for (int u = 0; u < 32; ++u) {
+            used[u] = w0 + 2 * u < nwg;
+            slot[u] = part_c + (used[u] ? (w0 + 2 * u) : 0) * W + k;
           }
-          ok = mailbox_wait<16>(slot, used, seq, error, spin_limit, v);
+          ok = mailbox_wait<32>(slot, used, seq, error, spin_limit, v);
 #pragma unroll
-          for (int u = 0; u < 16; ++u) s += v[u];
+          for (int u = 0; u < 32; ++u) s += v[u];
         }
       }
-      s_sum4[g][k] = s;
+      s_sum2[g][k] = s;
       if (tid < width && ok) {
         const unsigned long long* slot[1] = {piv_c + tid};
         const bool used[1] = {true};
@@ -393,104 +455,99 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
     }
     __syncthreads();
     if (s_fail) return;
-    if (tid < width) s_tot[tid] = (s_sum4[0][tid] + s_sum4[1][tid]) + (s_sum4[2][tid] + s_sum4[3][tid]);
+    if (tid < width) s_tot[tid] = s_sum2[0][tid] + s_sum2[1][tid];
     __syncthreads();
     if (tid < NB) {
+      // Householder on the compressed problem; lane k owns column k of the pivot rows and of G
       const int k = tid;
-      const T seen = s_scal[6];  // largest squared column norm of this panel so far (0 at its first column)
-      const Reflector h0 = make_reflector(s_piv[0], s_tot[0], kQrNegligible * seen);
-      T seen_next = fmaxf(seen, s_piv[0] * s_piv[0] + s_tot[0]);
-      const T tc0 = (k >= 1) ? h0.tau * (s_piv[k] + h0.scale * s_tot[k]) : T(0);
-      s_tc[0][k] = tc0;
-      if (k == 0) {
-        s_scal[0] = h0.scale; s_scal[1] = h0.beta; s_scal[2] = h0.tau;
+      T pv[S], g[S];
+#pragma unroll
+      for (int t = 0; t < S; ++t) {
+        pv[t] = (t < cols) ? s_piv[t * NB + k] : T(0);
+        g[t] = (t < cols) ? s_tot[t * NB + k] : T(0);
       }
-      T seen_out = seen_next;
-      if (pair) {
-        // row j+1 and the sums over the rows below it, after reflector j
-        const T q0 = s_piv[NB];                              // a_0[j+1]
-        const T v0_next = h0.scale * q0;                     // v[j+1]
-        const T tc0_1 = h0.tau * (s_piv[1] + h0.scale * s_tot[1]);
-        const T piv1 = s_piv[NB + k] - tc0 * v0_next;        // a'_k[j+1], k >= 1
-        const T sp_k = s_tot[k] - q0 * s_piv[NB + k];        // <a_0, a_k> below row j+1
-        const T sp_0 = s_tot[0] - q0 * q0;
-        const T sp_1 = s_tot[1] - q0 * s_piv[NB + 1];
-        const T u_k = s_tot[NB + k] - tc0 * h0.scale * sp_1 - tc0_1 * h0.scale * sp_k +
-                      tc0_1 * tc0 * h0.scale * h0.scale * sp_0;
-        // lane 1 holds the corrected squared norm of column j+1 below its pivot and its pivot entry
-        // (the last column of the matrix has nothing below its pivot: exactly zero, so tau = 0 as in LAPACK)
-        const T x2_1 = (j + 1 < n - 1) ? __shfl(u_k, 1, 64) : T(0), alpha1 = __shfl(piv1, 1, 64);
-        // size of the terms the corrected norm is the difference of (all three are >= 0 in exact arithmetic)
-        const T magnitude = s_tot[NB + 1] + T(2) * fabsf(tc0_1 * h0.scale * sp_1) +
-                            tc0_1 * tc0_1 * h0.scale * h0.scale * fabsf(sp_0);
-        const bool ok = (x2_1 - x2_1 == T(0)) && x2_1 >= kQrPairGuard * magnitude;  // finite and no cancellation
-        const Reflector h1 = make_reflector(alpha1, fmaxf(x2_1, T(0)), kQrNegligible * seen_next);
-        if (ok) seen_next = fmaxf(seen_next, alpha1 * alpha1 + fmaxf(x2_1, T(0)));
-        s_tc[1][k] = (k >= 2) ? h1.tau * (piv1 + h1.scale * u_k) : T(0);
-        seen_out = seen_next;
-        if (k == 0) {
-          s_scal[3] = h1.scale; s_scal[4] = h1.beta; s_scal[5] = h1.tau;
-          s_pair_ok = ok ? 1 : 0;
+      // for lane k < cols: size of the terms G[k][k] is made of (its own value, then every correction)
+      T size_diag = T(0);
+#pragma unroll
+      for (int t = 0; t < S; ++t)
+        if (k == t) size_diag = fabsf(g[t]);
+      T seen = s_seen;
+      int accepted = 0;
+#pragma unroll
+      for (int t = 0; t < S; ++t) {
+        if (t < cols && accepted == t) {
+          // column t = lane t: leading entry pv[t], the explicit rows below it, and G[t][t]
+          T explicit2 = T(0);
+#pragma unroll
+          for (int q = t + 1; q < S; ++q) explicit2 += pv[q] * pv[q];  // rows beyond `cols` hold zeros
+          const T alpha = round_lane_value(pv[t], t);
+          const T hidden2 = round_lane_value(g[t], t);
+          const T x2_explicit = round_lane_value(explicit2, t);
+          const T size_t_ = round_lane_value(size_diag, t);
+          // (the last column of the matrix has nothing below its pivot: exactly zero, so tau = 0 as in LAPACK)
+          const T x2 = (j + t < n - 1) ? x2_explicit + fmaxf(hidden2, T(0)) : T(0);
+          // The reflector is orthogonal to the accuracy of alpha^2 + x2; alpha and the explicit rows are
+          // exact, the hidden part carries an absolute error of about eps times the size of its terms.
+          const bool finite = hidden2 - hidden2 == T(0);
+          const bool ok = t == 0 || (finite && alpha * alpha + x2 >= kQrRoundGuard * size_t_);
+          if (ok) {
+            const Reflector h = make_reflector(alpha, x2, kQrNegligible * seen);
+            seen = fmaxf(seen, alpha * alpha + x2);
+            // d_k = <column t, column k> below pivot t
+            T d = g[t];
+#pragma unroll
+            for (int q = t + 1; q < S; ++q) d += round_lane_value(pv[q], t) * pv[q];
+            const T tc = (k > t) ? h.tau * (pv[t] + h.scale * d) : T(0);
+            s_tc[t][k] = tc;
+            if (k == 0) {
+              s_scal[t][0] = h.scale; s_scal[t][1] = h.beta; s_scal[t][2] = h.tau;
+            }
+            // explicit pivot rows below row t, then the Gram rows of the later columns of the round
+#pragma unroll
+            for (int q = t + 1; q < S; ++q) pv[q] -= tc * (h.scale * round_lane_value(pv[q], t));
+            const T g_tt = hidden2;
+#pragma unroll
+            for (int i = t + 1; i < S; ++i) {
+              const T g_it = round_lane_value(g[i], t);
+              const T tc_i = round_lane_value(tc, i);
+              const T first = tc * h.scale * g_it, second = tc_i * h.scale * g[t];
+              const T third = tc_i * tc * h.scale * h.scale * g_tt;
+              g[i] = g[i] - first - second + third;
+              if (k == i) size_diag += fabsf(first) + fabsf(second) + fabsf(third);
+            }
+            accepted = t + 1;
+          }
         }
-      } else if (k == 0) {
-        s_pair_ok = 0;
       }
-      // every lane read s_scal[6] above; lane 0 of the same wavefront may now replace it
-      if (k == 0) s_scal[6] = seen_out;
+      if (k == 0) {
+        s_accepted = accepted;
+        s_seen = seen;
+      }
     }
     __syncthreads();
-    const bool two = s_pair_ok != 0;
-    {
-      const T scale = s_scal[0], beta = s_scal[1], tauv = s_scal[2];
-      if (live && r >= j) {
-        if (r > j) {
-          const T v = a[0] * scale;
-          a[0] = v;
+    const int accepted = s_accepted;
 #pragma unroll
-          for (int k = 1; k < NB; ++k) a[k] -= s_tc[0][k] * v;
-        } else {
-          a[0] = beta;
+    for (int t = 0; t < S; ++t) {
+      if (t < accepted) {
+        const T scale = s_scal[t][0], beta = s_scal[t][1], tauv = s_scal[t][2];
+        const int jt = j + t;
+        // one instruction stream for the rows below the pivot (v = scaled entry), the pivot row
+        // (v = 1, entry <- beta) and the finished rows above it (v = 0)
+        const bool below = r > jt, pivot = r == jt;
+        const T v = below ? a[t] * scale : (pivot ? T(1) : T(0));
 #pragma unroll
-          for (int k = 1; k < NB; ++k) a[k] -= s_tc[0][k];
-          tau[j] = tauv;
+        for (int k = t + 1; k < NB; ++k) a[k] -= s_tc[t][k] * v;
+        a[t] = below ? v : (pivot ? beta : a[t]);
+        if (live && pivot) tau[jt] = tauv;
+        if (live) {
+          A[r + (int64_t)jt * lda] = a[t];  // column jt is final
+          vout[(r - vrow0) + (int64_t)(c + t) * ldv] = (r > jt) ? a[t] : (r == jt ? T(1) : T(0));
         }
       }
-      if (live) {
-        A[r + (int64_t)j * lda] = a[0];  // column j is final
-        vout[(r - vrow0) + (int64_t)c * ldv] = (r > j) ? a[0] : (r == j ? T(1) : T(0));
-      }
     }
-    if (two) {
-      const T scale = s_scal[3], beta = s_scal[4], tauv = s_scal[5];
-      const int j1 = j + 1;
-      if (live && r >= j1) {
-        if (r > j1) {
-          const T v = a[1] * scale;
-          a[1] = v;
-#pragma unroll
-          for (int k = 2; k < NB; ++k) a[k] -= s_tc[1][k] * v;
-        } else {
-          a[1] = beta;
-#pragma unroll
-          for (int k = 2; k < NB; ++k) a[k] -= s_tc[1][k];
-          tau[j1] = tauv;
-        }
-      }
-      if (live) {
-        A[r + (int64_t)j1 * lda] = a[1];
-        vout[(r - vrow0) + (int64_t)(c + 1) * ldv] = (r > j1) ? a[1] : (r == j1 ? T(1) : T(0));
-      }
-#pragma unroll
-      for (int k = 0; k + 2 < NB; ++k) a[k] = a[k + 2];
-      a[NB - 2] = T(0);
-      a[NB - 1] = T(0);
-      c += 2;
-    } else {
-#pragma unroll
-      for (int k = 0; k + 1 < NB; ++k) a[k] = a[k + 1];
-      a[NB - 1] = T(0);
-      c += 1;
-    }
+    // shift the row left by the number of finished columns
+    for (int q = 0; q < accepted; ++q) shift_left<1>(a);
+    c += accepted;
     // No barrier here: the shared arrays of the next round's first phase (s_wave, s_piv_out) were
     // last read before the barrier that follows the mailbox phase, and the arrays read above are
     // rewritten only behind the next such barrier, which every wavefront reaches after this point.
@@ -511,18 +568,6 @@ __global__ void extract_v_kernel(const T* __restrict__ A, int64_t lda, int nrows
     else v = A[(row0 + i) + (int64_t)(col0 + c) * lda];
     Vc[i + (int64_t)c * ldv] = v;
   }
-}
-
-// Value of `v` in lane `LANE` (a compile-time constant) as a wavefront-uniform scalar.
-template <int LANE>
-__device__ __forceinline__ float lane_value(float v) {
-  return __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)__float_as_uint(v), LANE));
-}
-template <int LANE>
-__device__ __forceinline__ double lane_value(double v) {
-  const int lo = __builtin_amdgcn_readlane(__double2loint(v), LANE);
-  const int hi = __builtin_amdgcn_readlane(__double2hiint(v), LANE);
-  return __hiloint2double(hi, lo);
 }
 
 // Column I of the factor, for I = 0 .. 31 by recursion: lane k holds row k of T in t[] and row k of
@@ -787,8 +832,8 @@ struct QrWorkspace {
   T* tau;     // n
   T* part;    // 2 x nwg x NB   partials of the launch-per-column fallback
   T* piv;     // 2 x NB
-  unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x 2 NB   mailboxes of the persistent panel kernel
-  unsigned long long* mail_piv;   // 2 x 2 NB
+  unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x kQrRoundMax NB   mailboxes of the persistent panel kernel
+  unsigned long long* mail_piv;   // 2 x kQrRoundMax NB
   unsigned* sync;  // [1] error flag of the persistent panel kernel
 };
 
@@ -802,8 +847,8 @@ static inline void qr_workspace_layout(WS& ws, int64_t n, QrWorkspace<T>* out) {
   q.tau = ws.template take<T>((size_t)n);
   q.part = ws.template take<T>((size_t)2 * nwg * kQrNb);
   q.piv = ws.template take<T>(2 * kQrNb);
-  q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * 2 * kQrNb);
-  q.mail_piv = ws.template take<unsigned long long>(2 * 2 * kQrNb);
+  q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * kQrRoundMax * kQrNb);
+  q.mail_piv = ws.template take<unsigned long long>(2 * kQrRoundMax * kQrNb);
   q.sync = ws.template take<unsigned>(64);
   if (out) *out = q;
 }
@@ -822,7 +867,7 @@ static inline size_t qr_workspace_bytes(int64_t n) {
 template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
                                        const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
-                                       unsigned spin_limit = kQrSpinLimit, int columns_per_round = 2) {
+                                       unsigned spin_limit = kQrSpinLimit, int columns_per_round = kQrRoundMax) {
   const int NB = kQrNb, OB = kBrMax;
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
@@ -832,7 +877,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
   hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
   {
     // mail_part and mail_piv are adjacent: one clear covers both (sequence number 0 = "nothing yet")
-    const int words = 2 * (2 * kQrPersistentMaxWg * 2 * kQrNb + 2 * 2 * kQrNb);
+    const int words = 2 * (2 * kQrPersistentMaxWg * kQrRoundMax * kQrNb + 2 * kQrRoundMax * kQrNb);
     hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3((words + 255) / 256), dim3(256), 0, s,
                        reinterpret_cast<unsigned*>(ws.mail_part), words);
   }
@@ -855,7 +900,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
                            ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
-                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, columns_per_round >= 2 ? 1 : 0);
+                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, columns_per_round);
         seq_base += (unsigned)nbw;
       } else {
         for (int j = p - 1; j < pe; ++j) {
