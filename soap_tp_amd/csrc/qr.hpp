@@ -529,19 +529,23 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
 #pragma unroll
     for (int t = 0; t < S; ++t) {
       if (t < accepted) {
-        const T scale = s_scal[t][0], beta = s_scal[t][1], tauv = s_scal[t][2];
+        const T scale = s_scal[t][0], tauv = s_scal[t][2];
         const int jt = j + t;
         // one instruction stream for the rows below the pivot (v = scaled entry), the pivot row
-        // (v = 1, entry <- beta) and the finished rows above it (v = 0)
+        // (v = 1) and the finished rows above it (v = 0)
         const bool below = r > jt, pivot = r == jt;
         const T v = below ? a[t] * scale : (pivot ? T(1) : T(0));
 #pragma unroll
         for (int k = t + 1; k < NB; ++k) a[k] -= s_tc[t][k] * v;
-        a[t] = below ? v : (pivot ? beta : a[t]);
         if (live && pivot) tau[jt] = tauv;
         if (live) {
-          A[r + (int64_t)jt * lda] = a[t];  // column jt is final
-          vout[(r - vrow0) + (int64_t)(c + t) * ldv] = (r > jt) ? a[t] : (r == jt ? T(1) : T(0));
+          // Column jt is final.  Both copies get the reflector in clean form (unit diagonal, zeros
+          // above it inside the panel's square top block): the entries of R on and above the
+          // diagonal of that block are dropped, the factorisation has no reader for them, and the
+          // panel's columns in A can then stand in for V in V^T [V | rest of the block].
+          const T vclean = below ? v : (pivot ? T(1) : T(0));
+          A[r + (int64_t)jt * lda] = vclean;
+          vout[(r - vrow0) + (int64_t)(c + t) * ldv] = vclean;
         }
       }
     }
@@ -597,12 +601,21 @@ struct LarftColumn {
 // of a wider factor are built by one launch.  Everything stays in registers: the recursion over
 // the columns is unrolled at compile time and values cross lanes as scalars (v_readlane).
 // Reflectors beyond the block's width count as tau = 0, which leaves their rows and columns zero.
-// G may arrive as `splits` unreduced split-K slices (`slab` elements apart), summed while loading.
+// G may arrive as `splits` unreduced split-K slices (`slab` elements apart), summed while loading:
+// the block's 32 (double: 4) groups of 32 threads take slices z = group, group + groups, ... (all
+// loads of a thread are in flight together), and the groups' sums are then added in a fixed order through LDS.
 template <typename T>
-__global__ __launch_bounds__(128) void larft32_kernel(const T* __restrict__ G, int ldg, int splits, int64_t slab,
-                                                       const T* __restrict__ tau, int nbw, T* __restrict__ Tm,
-                                                       int ldt) {
-  __shared__ T s_g[4][32][33];
+constexpr int larft_groups() {
+  return sizeof(T) == 8 ? 4 : 32;  // double (already summed input only): 128 threads, all registers for the recursion
+}
+
+template <typename T>
+__global__ __launch_bounds__(32 * larft_groups<T>()) void larft32_kernel(const T* __restrict__ G, int ldg, int splits,
+                                                                    int64_t slab, const T* __restrict__ tau, int nbw,
+                                                                    T* __restrict__ Tm, int ldt) {
+  constexpr int STAGE = sizeof(T) == 8 ? 4 : 8;  // groups that exchange through LDS at a time (33 KB)
+  constexpr int kLarftGroups = larft_groups<T>();
+  __shared__ T s_g[STAGE][32][33];
   const int b = blockIdx.x;
   const int w = min(32, nbw - 32 * b);
   G += (int64_t)32 * b * (ldg + 1);
@@ -610,25 +623,39 @@ __global__ __launch_bounds__(128) void larft32_kernel(const T* __restrict__ G, i
   tau += 32 * b;
   const int k = threadIdx.x & 31, zg = threadIdx.x >> 5;
   T t[32], g[32];
-  // slices z = zg, zg + 4, ... are summed by slice group zg (128 threads = 4 groups), the groups then
-  // in a fixed order
 #pragma unroll
   for (int c = 0; c < 32; ++c) g[c] = T(0);
   if (k < w) {
-    for (int z = zg; z < splits; z += 4) {
+    for (int z = zg; z < splits; z += kLarftGroups) {
       const T* slice = G + (int64_t)z * slab + k;
 #pragma unroll
       for (int c = 0; c < 32; ++c) g[c] += (c < w) ? slice[c * ldg] : T(0);
     }
   }
   if (splits > 1) {
+    // groups STAGE .. 31 hand their sums to groups 0 .. STAGE-1, STAGE groups at a time
+    for (int base = STAGE; base < kLarftGroups && base < splits; base += STAGE) {
+      if (zg >= base && zg < base + STAGE) {
 #pragma unroll
-    for (int c = 0; c < 32; ++c) s_g[zg][k][c] = g[c];
+        for (int c = 0; c < 32; ++c) s_g[zg - base][k][c] = g[c];
+      }
+      __syncthreads();
+      if (zg < STAGE && zg + base < splits) {
+#pragma unroll
+        for (int c = 0; c < 32; ++c) g[c] += s_g[zg][k][c];
+      }
+      __syncthreads();
+    }
+    if (zg > 0 && zg < STAGE) {
+#pragma unroll
+      for (int c = 0; c < 32; ++c) s_g[zg][k][c] = g[c];
+    }
     __syncthreads();
     if (zg == 0) {
+      for (int q = 1; q < STAGE && q < splits; ++q) {
 #pragma unroll
-      for (int c = 0; c < 32; ++c)
-        g[c] = (s_g[0][k][c] + s_g[1][k][c]) + (s_g[2][k][c] + s_g[3][k][c]);
+        for (int c = 0; c < 32; ++c) g[c] += s_g[q][k][c];
+      }
     }
   }
   if (threadIdx.x >= 64) return;  // the recursion runs in the first wavefront; its lanes 32..63 carry zeros
@@ -709,7 +736,7 @@ static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws
   using Skinny = typename SkinnyTile<T>::type;
   const int blocks = (int)ceil_div64(nbw, 32);
   if (first_block < blocks) {
-    hipLaunchKernelGGL((larft32_kernel<T>), dim3(blocks - first_block), dim3(128), 0, s,
+    hipLaunchKernelGGL((larft32_kernel<T>), dim3(blocks - first_block), dim3(32 * larft_groups<T>()), 0, s,
                        ws.gram + (int64_t)32 * first_block * (kBrMax + 1), kBrMax, 1, (int64_t)0, tau + 32 * first_block,
                        nbw - 32 * first_block, Tm + (int64_t)32 * first_block * (kBrMax + 1), kBrMax);
     SOAPMI_LAUNCH_CHECK();
@@ -764,6 +791,81 @@ __global__ __launch_bounds__(256) void reflector_w2_kernel(const T* __restrict__
       acc += s_t[l][q] * ((s_w[cc][0][q] + s_w[cc][1][q]) + (s_w[cc][2][q] + s_w[cc][3][q]));
     W2[l + (int64_t)c * ldw2] = acc;
   }
+}
+
+// W2 (M x N, ld ldw2) = T^T W for a panel of M <= 32 reflectors without forming T: the inverse of the
+// compact-WY factor is known in closed form, T^-1 = strict upper triangle of V^T V + diag(1 / tau),
+// so T^T W is the solution X of a lower triangular system, x_i = tau_i (w_i - sum_{l<i} G[l][i] x_l).
+// `part` holds the split-K slices of V^T [V | C] (M rows, ld M): columns 0..M-1 are G = V^T V,
+// column M + c is column c of W = V^T C.  A reflector with tau = 0 (none) gets x_i = 0, as its
+// zero row and column of T would give.  256 threads = 8 groups of 32 lanes, one column of W per
+// group: everyone sums G's slices into LDS (fixed order), each group sums and substitutes its column.
+constexpr int kW2SolveCols = 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void reflector_w2_solve_kernel(const T* __restrict__ part, int splits, int64_t slab,
+                                                                 int M, int N, const T* __restrict__ tau,
+                                                                 T* __restrict__ W2, int ldw2) {
+  __shared__ T s_g[32][33];
+  const int tid = threadIdx.x, l = tid & 31, group = tid >> 5;
+  const int c = blockIdx.x * kW2SolveCols + group;
+  {
+    // entry e = tid + 256 q of the M x M block G (column-major, ld M); out-of-range entries read
+    // element 0 and are zeroed afterwards, so that the loads carry no branch
+    int offset[4];
+    bool inside[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = tid + 256 * q, row = e & 31, col = e >> 5;
+      inside[q] = row < M && col < M;
+      offset[q] = inside[q] ? row + col * M : 0;
+    }
+    T g[4] = {T(0), T(0), T(0), T(0)};
+    int z = 0;
+    for (; z + 8 <= splits; z += 8) {
+      T v[8][4];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[u][q] = part[(int64_t)(z + u) * slab + offset[q]];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) g[q] += v[u][q];
+    }
+    for (; z < splits; ++z)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) g[q] += part[(int64_t)z * slab + offset[q]];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = tid + 256 * q;
+      s_g[e & 31][e >> 5] = inside[q] ? g[q] : T(0);
+    }
+  }
+  const bool mine = l < M && c < N;
+  T w = T(0);
+  {
+    const T* column = part + (mine ? l + (int64_t)(M + c) * M : 0);
+    int z = 0;
+    for (; z + 8 <= splits; z += 8) {
+      T v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = column[(int64_t)(z + u) * slab];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) w += v[u];
+    }
+    for (; z < splits; ++z) w += column[(int64_t)z * slab];
+    if (!mine) w = T(0);
+  }
+  __syncthreads();
+  const T tau_l = (l < M) ? tau[l] : T(0);
+  T x = T(0);
+  for (int i = 0; i < M; ++i) {
+    const T xi = __shfl(tau_l * w, i, 32);  // final for lane i: every l < i has been subtracted
+    if (l == i) x = xi;
+    if (l > i) w -= s_g[i][l] * xi;
+  }
+  if (mine) W2[l + (int64_t)c * ldw2] = x;
 }
 
 template <typename T>
@@ -911,15 +1013,32 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
         v_written = false;
       }
       SOAPMI_LAUNCH_CHECK();
-      if (pe < PE) {  // the panel's reflectors act on the rest of the outer block only
+      if (pe < PE && v_written) {
+        // The panel's reflectors act on the rest of the outer block only.  One product gives the
+        // slices of V^T [V | C] (the panel's own columns of A hold V in clean form); the middle
+        // factor T^T is applied as a triangular solve with V^T V, so no T is needed here: the
+        // diagonal blocks of the outer factor are all built after the block's last panel.
+        using Skinny = typename SkinnyTile<T>::type;
+        const int ncols = PE - p, nc = PE - pe;
+        int slices = 1;
+        rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, ncols, rows, inner.v, ldv, A + p + (int64_t)p * lda, lda,
+                                         split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
+                                         ws.br.splitk, &slices);
+        if (rc) return rc;
+        hipLaunchKernelGGL((reflector_w2_solve_kernel<T>), dim3((unsigned)ceil_div64(nc, kW2SolveCols)), dim3(256), 0, s,
+                           ws.br.splitk, slices, (int64_t)nbw * ncols, nbw, nc, ws.tau + p, ws.br.w2, kBrMax);
+        SOAPMI_LAUNCH_CHECK();
+        rc = gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), inner.v, ldv, ws.br.w2, kBrMax, T(1), A + p + (int64_t)pe * lda, lda);
+        if (rc) return rc;
+      } else if (pe < PE) {
         T* Tin = Tm + (int64_t)(p - P) * (OB + 1);  // diagonal block of the outer factor
-        if (!v_written) launch_extract_v<T>(s, A, lda, rows, p, p, nbw, inner.v, ldv);
+        launch_extract_v<T>(s, A, lda, rows, p, p, nbw, inner.v, ldv);
         int slices = 1;  // V^T V stays in split-K slices; the factor kernel sums them while loading
         rc = gemm_to_partials<T, typename SkinnyTile<T>::type>(s, 1, 0, nbw, nbw, rows, inner.v, ldv, inner.v, ldv,
                                                                split_count(1, rows, nbw, nbw, ldv), inner.splitk,
                                                                &slices);
         if (rc) return rc;
-        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(128), 0, s, inner.splitk, nbw, slices,
+        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(32 * larft_groups<T>()), 0, s, inner.splitk, nbw, slices,
                            (int64_t)nbw * nbw, ws.tau + p, nbw, Tin, OB);
         SOAPMI_LAUNCH_CHECK();
         rc = apply_block_reflector<T>(s, inner, Tin, true, rows, nbw, PE - pe, ldv, A + p + (int64_t)pe * lda, lda);
