@@ -392,6 +392,17 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_batched_kernel(const BatchedGemm
   gemm_tile_body<T, Cfg, EpiStore<T>, -1>(b.p, b.e, blockIdx.x, 0);
 }
 
+// The same product for blockIdx.z = 0 .. batch-1, with the operands and the result a fixed number of
+// elements further on each time (general path: any size and alignment).
+template <typename T, class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void gemm_strided_kernel(GemmProblem<T> p, EpiStore<T> e, int64_t stride_a,
+                                                               int64_t stride_b, int64_t stride_c) {
+  p.A += (int64_t)blockIdx.z * stride_a;
+  p.B += (int64_t)blockIdx.z * stride_b;
+  e.C += (int64_t)blockIdx.z * stride_c;
+  gemm_tile_body<T, Cfg, EpiStore<T>, -1>(p, e, blockIdx.x, 0);
+}
+
 // Device-side twin of make_problem for the default tile.
 template <typename T, class Cfg>
 __device__ __forceinline__ void fill_batched(BatchedGemm<T>& b, int transA, int transB, int M, int N, int K,
@@ -541,6 +552,25 @@ static inline int gemm(hipStream_t stream, int transA, int transB, int M, int N,
   }
   EpiStore<T> ep{C, ldc, alpha, beta};
   return launch_gemm<T, EpiStore<T>, Cfg>(stream, p, ep, 1);
+}
+
+// C_b = alpha * A_b * B_b + beta * C_b for b = 0 .. batch-1 in one launch (no transposes); operand b
+// starts b * stride elements after operand 0.
+template <typename T, class Cfg>
+static inline int gemm_strided_batch(hipStream_t stream, int M, int N, int K, T alpha, const T* A, int64_t lda,
+                                     int64_t stride_a, const T* B, int64_t ldb, int64_t stride_b, T beta, T* C,
+                                     int64_t ldc, int64_t stride_c, int batch) {
+  if (M <= 0 || N <= 0 || batch <= 0) return kOk;
+  constexpr int VW = Vec16<T>::W;
+  GemmProblem<T> p = make_problem<T, Cfg>(0, 0, M, N, K, A, lda, B, ldb, false);
+  p.vecA = p.vecA && stride_a % VW == 0;
+  p.vecB = p.vecB && stride_b % VW == 0;
+  EpiStore<T> ep{C, ldc, alpha, beta};
+  const int chunk = (p.num_tiles + 7) / 8;
+  hipLaunchKernelGGL((gemm_strided_kernel<T, Cfg>), dim3(8 * chunk, 1, batch), dim3(Cfg::NT), 0, stream, p, ep, stride_a,
+                     stride_b, stride_c);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
 }
 
 // op(A) op(B) cut into K slices whose partial products stay unreduced in `partials` (slice z at

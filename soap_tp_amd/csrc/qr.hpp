@@ -728,12 +728,14 @@ static inline void block_reflector_layout(WS& ws, int64_t n, BlockReflectorWs<T>
 
 // T (ld kBrMax) from G = V^T V (in ws.gram, ld kBrMax) and tau for nbw <= kBrMax reflectors.  The
 // diagonal 32-blocks [first_block, ...) come from larft32_kernel (earlier ones are already in Tm,
-// the rest of Tm must be zero); block column j then follows from the blocks to its left:
-//   T[0:R, j] = -T[0:R, 0:R] (G[0:R, j] T[j, j]),  R = 32 j.
+// the rest of Tm must be zero).  The blocks above the diagonal follow by doubling: two neighbouring
+// spans of S reflectors with factors T11 and T22 have the joint factor [T11 T12; 0 T22] with
+// T12 = -T11 (G12 T22); all pairs of one span length are independent and share a launch, so a
+// 256-wide factor takes three levels (S = 32, 64, 128) of two products each.
 template <typename T>
 static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws, int nbw, const T* tau, T* Tm,
                                     int first_block) {
-  using Skinny = typename SkinnyTile<T>::type;
+  using Small = typename SmallTile<T>::type;
   const int blocks = (int)ceil_div64(nbw, 32);
   if (first_block < blocks) {
     hipLaunchKernelGGL((larft32_kernel<T>), dim3(blocks - first_block), dim3(32 * larft_groups<T>()), 0, s,
@@ -741,13 +743,27 @@ static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws
                        nbw - 32 * first_block, Tm + (int64_t)32 * first_block * (kBrMax + 1), kBrMax);
     SOAPMI_LAUNCH_CHECK();
   }
-  for (int j = 1; j < blocks; ++j) {
-    const int R = 32 * j, wj = std::min(32, nbw - R);
-    int rc = gemm<T, Skinny>(s, 0, 0, R, wj, wj, T(1), ws.gram + (int64_t)R * kBrMax, kBrMax,
-                             Tm + (int64_t)R * (kBrMax + 1), kBrMax, T(0), ws.mx, kBrMax);
+  for (int S = 32; S < nbw; S *= 2) {
+    const int64_t pair_stride = (int64_t)2 * S * (kBrMax + 1);  // from one pair's blocks to the next pair's
+    const int64_t off12 = (int64_t)S * kBrMax;                  // block (0, S) of a pair, relative to its block (0, 0)
+    const int64_t off22 = (int64_t)S * (kBrMax + 1);
+    const int full = nbw / (2 * S);                             // pairs whose right span is complete
+    const int right = nbw - (2 * S * full + S);                 // width of the last, shorter right span (<= 0: none)
+    int rc = gemm_strided_batch<T, Small>(s, S, S, S, T(1), ws.gram + off12, kBrMax, pair_stride, Tm + off22, kBrMax,
+                                          pair_stride, T(0), ws.mx + off12, kBrMax, pair_stride, full);
     if (rc) return rc;
-    rc = gemm<T, Skinny>(s, 0, 0, R, wj, R, T(-1), Tm, kBrMax, ws.mx, kBrMax, T(0), Tm + (int64_t)R * kBrMax, kBrMax);
+    rc = gemm_strided_batch<T, Small>(s, S, S, S, T(-1), Tm, kBrMax, pair_stride, ws.mx + off12, kBrMax, pair_stride,
+                                      T(0), Tm + off12, kBrMax, pair_stride, full);
     if (rc) return rc;
+    if (right > 0) {
+      const int64_t base = (int64_t)full * pair_stride;
+      rc = gemm<T, Small>(s, 0, 0, S, right, right, T(1), ws.gram + base + off12, kBrMax, Tm + base + off22, kBrMax, T(0),
+                          ws.mx + base + off12, kBrMax);
+      if (rc) return rc;
+      rc = gemm<T, Small>(s, 0, 0, S, right, S, T(-1), Tm + base, kBrMax, ws.mx + base + off12, kBrMax, T(0),
+                          Tm + base + off12, kBrMax);
+      if (rc) return rc;
+    }
   }
   return kOk;
 }
