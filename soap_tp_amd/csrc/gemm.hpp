@@ -510,8 +510,10 @@ static inline int launch_gemm(hipStream_t stream, const GemmProblem<T>& p, const
   if (p.M <= 0 || p.N <= 0) return kOk;
   const int chunk = (p.num_tiles + 7) / 8;
   dim3 grid(8 * chunk, k_splits, 1);
+  // (K slices start at multiples of k_chunk, so with K and k_chunk multiples of the slab every
+  // slice, a shorter last one included, is a whole number of slabs)
   const bool fast = p.vecA && p.vecB && p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K > 0 &&
-                    p.K % Cfg::BK == 0 && p.k_chunk % Cfg::BK == 0 && p.K % p.k_chunk == 0;
+                    p.K % Cfg::BK == 0 && p.k_chunk % Cfg::BK == 0;
   const int mode = fast ? ((p.transA ? 0 : 1) | (p.transB ? 2 : 0)) : -1;
   switch (mode) {
     case 0: hipLaunchKernelGGL((gemm_kernel<T, Cfg, Epi, 0>), grid, dim3(Cfg::NT), 0, stream, p, epi); break;

@@ -769,14 +769,27 @@ static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws
 }
 
 // Number of K slices for a tall-skinny product with `tiles` output tiles, K = rows, an M x N
-// output: enough slices to occupy the chip (about 512 workgroups), at least 128 rows each, and no
-// more partial results than the split-K buffer (kBrSplits * kBrMax * ldv elements) holds.
+// output.  Slices have at least 128 rows and the partial results must fit the split-K buffer
+// (kBrSplits * kBrMax * ldv elements).  With a handful of tiles: as many slices as it takes to
+// occupy the chip (about 512 workgroups).  With more tiles the workgroups of a launch are spread
+// over the 256 CUs and a CU works through its share one after the other, so the time goes as
+// ceil(tiles * slices / 256) / slices: the slice count that minimises it is taken (fewest slices
+// among near-equal ones), which avoids launches whose last CU round is nearly empty.
 static inline int split_count(int64_t tiles, int rows, int M, int N, int64_t ldv) {
   if (rows < 512) return 1;
-  int64_t splits = std::min<int64_t>(ceil_div64(512, tiles), rows / 128);
   const int64_t capacity = (int64_t)kBrSplits * kBrMax * ldv / std::max<int64_t>(1, (int64_t)M * N);
-  splits = std::min<int64_t>(splits, std::min<int64_t>(capacity, 64));
-  return (int)std::max<int64_t>(splits, 1);
+  const int64_t most = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(capacity, 64), rows / 128));
+  if (tiles <= 8) return (int)std::min<int64_t>(ceil_div64(512, tiles), most);
+  int best = 1;
+  double best_cost = (double)ceil_div64(tiles, 256);
+  for (int64_t slices = 2; slices <= std::min<int64_t>(most, 16); ++slices) {
+    const double cost = (double)ceil_div64(tiles * slices, 256) / (double)slices;
+    if (cost < 0.97 * best_cost) {
+      best = (int)slices;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 // W2 (M x N, ld ldw2) = op(T) * (sum of the split-K slices of W), M <= 32: the middle product of a
