@@ -176,6 +176,18 @@ def test_qr_launch_per_column_panel_path(size, device):
         _native.call("soapmi_set_option", b"qr_persistent_max_workgroups", 129)
 
 
+@pytest.mark.parametrize("size", [289, 545, 1000])
+def test_qr_block_reflector_widths(size, device):
+    """Sizes whose last 256-column block reflector has a width that is no multiple of 32, 64 or 128:
+    the factor T of such a block is assembled from unequal spans (33 = 32 + 1, 232 = 128 + 64 + 32 + 8)."""
+    matrix = make_matrix(size, size, seed=SEED + 17 * size)
+    factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+    ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
+    expected_q = oracle.householder_qr(matrix)
+    assert relative_l2(factor, expected_q) <= 5e-5
+    torch.testing.assert_close(factor.T @ factor, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("kind", ["paired_columns", "graded", "rank_deficient", "repeated_column"])
 @pytest.mark.parametrize("columns_per_round", [1, 2, 3, 4])
 def test_qr_is_backward_stable_on_hard_matrices(kind, columns_per_round, device):
