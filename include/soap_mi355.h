@@ -54,6 +54,10 @@ const char* soapmi_last_error(void);
  *       the reflectors after the first follow from those by rank-one corrections (guarded: a
  *       column whose corrected norm shows cancellation ends the round and starts the next one with
  *       directly computed sums); 1 computes every column's sums directly.
+ *   "refresh_streams"  1 or 2 (default 2): with 2, soapmi_refresh_f32 runs the left and the right
+ *       factorisation chain side by side, the smaller one on a stream the library owns, forked from
+ *       and joined back into the caller's stream with events; with 1 everything is enqueued on the
+ *       caller's stream, one chain after the other.  The results are the same bit for bit.
  *   "message_spin_limit"  0..4194304 (default 4194304): how many times a workgroup of the QR panel
  *       kernel or of the tridiagonalisation's column kernel polls for another workgroup's message
  *       before it gives up.  Giving up never hangs and never passes silently: the kernels leave,

@@ -36,6 +36,8 @@ static std::atomic<int> g_qr_persistent_max_wg{kQrPersistentMaxWg};
 static std::atomic<unsigned> g_message_spin_limit{kQrSpinLimit};
 // panel columns the QR factors per message round (see soapmi_set_option)
 static std::atomic<int> g_qr_columns_per_round{kQrRoundMax};
+// streams a basis refresh uses: 2 = the two factorisation chains side by side, 1 = one after the other
+static std::atomic<int> g_refresh_streams{2};
 static std::mutex g_scratch_mutex;
 
 static int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out) {
@@ -167,6 +169,11 @@ int soapmi_set_option(const char* name, int64_t value) {
   if (strcmp(name, "message_spin_limit") == 0) {
     SOAPMI_REQUIRE(value >= 0 && value <= (int64_t)kQrSpinLimit, "message_spin_limit must be in 0..%u", kQrSpinLimit);
     g_message_spin_limit.store((unsigned)value);
+    return kOk;
+  }
+  if (strcmp(name, "refresh_streams") == 0) {
+    SOAPMI_REQUIRE(value == 1 || value == 2, "refresh_streams must be 1 or 2");
+    g_refresh_streams.store((int)value);
     return kOk;
   }
   set_error("unknown option '%s'", name);
@@ -597,20 +604,26 @@ int soapmi_refresh_f32(float* momentum, int64_t ldm, float* variance, int64_t ld
   if (rc) return rc;
   // fork: the smaller chain goes to the side stream, whose latency-bound panel kernels fill the
   // gaps of the larger one
+  const bool two_streams = g_refresh_streams.load() == 2;
   const bool left_on_side = rows <= cols;
-  SOAPMI_HIP(hipEventRecord(side->fork, main_stream));
-  SOAPMI_HIP(hipStreamWaitEvent(side->stream, side->fork, 0));
+  void* const side_or_main = two_streams ? (void*)side->stream : stream;
+  if (two_streams) {
+    SOAPMI_HIP(hipEventRecord(side->fork, main_stream));
+    SOAPMI_HIP(hipStreamWaitEvent(side->stream, side->fork, 0));
+  }
   int rc_left = soapmi_power_iteration_qr_f32(left_preconditioner, q_left, left_work, rows, ldl, ldql, ldlw, symmetrize,
                                               left_order, nullptr, left_ws, left_bytes,
-                                              left_on_side ? (void*)side->stream : stream);
+                                              left_on_side ? side_or_main : stream);
   int rc_right = kOk;
   if (rc_left == kOk)
     rc_right = soapmi_power_iteration_qr_f32(right_preconditioner, q_right, right_work, cols, ldr, ldqr, ldrw,
                                              symmetrize, right_order, nullptr, right_ws, right_bytes,
-                                             left_on_side ? stream : (void*)side->stream);
+                                             left_on_side ? stream : side_or_main);
   // join, also after a failure: nothing may stay detached from the caller's stream
-  SOAPMI_HIP(hipEventRecord(side->join, side->stream));
-  SOAPMI_HIP(hipStreamWaitEvent(main_stream, side->join, 0));
+  if (two_streams) {
+    SOAPMI_HIP(hipEventRecord(side->join, side->stream));
+    SOAPMI_HIP(hipStreamWaitEvent(main_stream, side->join, 0));
+  }
   if (rc_left) return rc_left;
   if (rc_right) return rc_right;
   rc = soapmi_permute_f32(variance, ldv, rows, cols, left_order, right_order, ws, need, stream);

@@ -72,12 +72,15 @@ static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, i
   const int64_t ldv = n;
   for (int bi = blocks - 1; bi >= 0; --bi) {
     const int p = bi * OB, pe = std::min(nref, p + OB), nbw = pe - p;
-    const int rows = n - p - 1;
-    launch_extract_v<T>(s, A, lda, rows, p + 1, p, nbw, ws.br.v, ldv);
+    // The block's reflectors start in row p + 1; row p (all zero in V) is carried along so that the
+    // products' row extent n - p stays a multiple of the MFMA tile whenever n and the block width are
+    // (the fast product path), instead of one short of it.
+    const int rows = n - p;
+    launch_extract_v<T>(s, A, lda, rows, p, p, nbw, ws.br.v, ldv, 1);
     SOAPMI_LAUNCH_CHECK();
     rc = build_t_factor<T>(s, ws.br, rows, nbw, ldv, ws.tau + p, ws.t_block);
     if (rc) return rc;
-    rc = apply_block_reflector<T>(s, ws.br, ws.t_block, false, rows, nbw, n, ldv, Z + (p + 1), ldz);
+    rc = apply_block_reflector<T>(s, ws.br, ws.t_block, false, rows, nbw, n, ldv, Z + p, ldz);
     if (rc) return rc;
   }
   hipLaunchKernelGGL((eigh_poison_on_error_kernel<T>), dim3((unsigned)ceil_div64(n, 256)), dim3(256), 0, s, w, Z, ldz, n,

@@ -558,17 +558,19 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
   }
 }
 
-// Vc (nrows x nbw, ld ldv) <- the unit-lower-trapezoidal reflector block stored in A with its
-// unit diagonal at (row0 + c, col0 + c): zeros above, ones on, A below.
+// Vc (nrows x nbw, ld ldv) <- the unit-lower-trapezoidal reflector block stored in A, column c with
+// its unit entry in row c + shift of the block: zeros above, one there, A[row0 + i, col0 + c] below.
+// shift = 0: QR reflectors (unit diagonal at (row0 + c, col0 + c)); shift = 1: the reflectors of a
+// tridiagonalisation, which start one row below the diagonal (row 0 of the block is then all zero).
 template <typename T>
 __global__ void extract_v_kernel(const T* __restrict__ A, int64_t lda, int nrows, int row0, int col0, int nbw,
-                                 T* __restrict__ Vc, int64_t ldv) {
+                                 T* __restrict__ Vc, int64_t ldv, int shift) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;  // row within the block
   if (i >= nrows) return;
   for (int c = blockIdx.y; c < nbw; c += gridDim.y) {
     T v;
-    if (i < c) v = T(0);
-    else if (i == c) v = T(1);
+    if (i < c + shift) v = T(0);
+    else if (i == c + shift) v = T(1);
     else v = A[(row0 + i) + (int64_t)(col0 + c) * lda];
     Vc[i + (int64_t)c * ldv] = v;
   }
@@ -950,9 +952,9 @@ static inline int apply_block_reflector(hipStream_t s, const BlockReflectorWs<T>
 
 template <typename T>
 static inline void launch_extract_v(hipStream_t s, const T* A, int64_t lda, int rows, int row0, int col0, int nbw,
-                                    T* V, int64_t ldv) {
+                                    T* V, int64_t ldv, int shift = 0) {
   hipLaunchKernelGGL((extract_v_kernel<T>), dim3((unsigned)ceil_div64(rows, 256), (unsigned)std::min(nbw, 32)),
-                     dim3(256), 0, s, A, lda, rows, row0, col0, nbw, V, ldv);
+                     dim3(256), 0, s, A, lda, rows, row0, col0, nbw, V, ldv, shift);
 }
 
 // ---- QR driver -------------------------------------------------------------------------------

@@ -3,6 +3,8 @@
 //   abi_probe [rows cols [repeats [copies]]]
 //   abi_probe qr n          QR of a pseudo-random n x n matrix (library-owned workspace), Q checked on the host
 //   abi_probe eigh n        fp64 eigendecomposition of a symmetric n x n matrix, checked on the host
+//   abi_probe qr|eigh n timed   the same call four times, the last three timed, no host check (the
+//                               check is cubic on one core: minutes at n = 11008)
 //
 // 1. `copies` layout copies of a rows x cols fp32 matrix (4*rows*cols bytes read, as many written):
 //    the kernel of known size that hardware-counter readings of a profiled run are scaled by.
@@ -49,8 +51,10 @@ static float host_value(uint64_t index) {
   return (float)((double)(x & 0xFFFFFF) / (double)0x1000000 - 0.5);
 }
 
-// Q^T Q = I and Q^T A upper triangular for soapmi_qr_f32 with a NULL workspace.
-static int check_qr(int64_t n) {
+// Q^T Q = I and Q^T A upper triangular for soapmi_qr_f32 with a NULL workspace.  With timed_only the
+// (cubic, single-threaded) host check is left out and the call is repeated between two events: the
+// form a profiler run uses at large n.
+static int check_qr(int64_t n, bool timed_only) {
   std::vector<float> a((size_t)n * n), q((size_t)n * n);
   for (size_t i = 0; i < a.size(); ++i) a[i] = host_value(i + 17);
   float *d_a, *d_q;
@@ -59,6 +63,26 @@ static int check_qr(int64_t n) {
   HIP_OK(hipMemcpy(d_a, a.data(), a.size() * sizeof(float), hipMemcpyHostToDevice));
   ABI_OK(soapmi_qr_f32(d_a, d_q, n, n, n, nullptr, 0, nullptr));
   HIP_OK(hipDeviceSynchronize());
+  if (timed_only) {
+    hipEvent_t start, stop;
+    HIP_OK(hipEventCreate(&start));
+    HIP_OK(hipEventCreate(&stop));
+    float total_ms = 0.0f;
+    const int repeats = 3;
+    for (int i = 0; i < repeats; ++i) {
+      HIP_OK(hipMemcpy(d_a, a.data(), a.size() * sizeof(float), hipMemcpyHostToDevice));
+      HIP_OK(hipEventRecord(start, nullptr));
+      ABI_OK(soapmi_qr_f32(d_a, d_q, n, n, n, nullptr, 0, nullptr));
+      HIP_OK(hipEventRecord(stop, nullptr));
+      HIP_OK(hipEventSynchronize(stop));
+      float ms = 0.0f;
+      HIP_OK(hipEventElapsedTime(&ms, start, stop));
+      total_ms += ms;
+    }
+    std::printf("qr n=%lld: %.3f ms per call (mean of %d)\n", (long long)n, total_ms / repeats, repeats);
+    hipFree(d_a); hipFree(d_q);
+    return 0;
+  }
   HIP_OK(hipMemcpy(q.data(), d_q, q.size() * sizeof(float), hipMemcpyDeviceToHost));
   double worst_orth = 0.0, worst_lower = 0.0;
   for (int64_t i = 0; i < n; ++i)
@@ -80,7 +104,7 @@ static int check_qr(int64_t n) {
 }
 
 // A Z = Z diag(w), Z^T Z = I, w ascending for soapmi_eigh_f64 with a NULL workspace.
-static int check_eigh(int64_t n) {
+static int check_eigh(int64_t n, bool timed_only) {
   std::vector<double> a((size_t)n * n), z((size_t)n * n), w((size_t)n);
   for (int64_t i = 0; i < n; ++i)
     for (int64_t j = 0; j <= i; ++j) a[i + j * n] = a[j + i * n] = host_value((uint64_t)(i * n + j) + 5);
@@ -91,6 +115,26 @@ static int check_eigh(int64_t n) {
   HIP_OK(hipMemcpy(d_a, a.data(), a.size() * sizeof(double), hipMemcpyHostToDevice));
   ABI_OK(soapmi_eigh_f64(d_a, d_w, d_z, n, n, n, nullptr, 0, nullptr));
   HIP_OK(hipDeviceSynchronize());
+  if (timed_only) {
+    hipEvent_t start, stop;
+    HIP_OK(hipEventCreate(&start));
+    HIP_OK(hipEventCreate(&stop));
+    float total_ms = 0.0f;
+    const int repeats = 3;
+    for (int i = 0; i < repeats; ++i) {
+      HIP_OK(hipMemcpy(d_a, a.data(), a.size() * sizeof(double), hipMemcpyHostToDevice));
+      HIP_OK(hipEventRecord(start, nullptr));
+      ABI_OK(soapmi_eigh_f64(d_a, d_w, d_z, n, n, n, nullptr, 0, nullptr));
+      HIP_OK(hipEventRecord(stop, nullptr));
+      HIP_OK(hipEventSynchronize(stop));
+      float ms = 0.0f;
+      HIP_OK(hipEventElapsedTime(&ms, start, stop));
+      total_ms += ms;
+    }
+    std::printf("eigh n=%lld: %.3f ms per call (mean of %d)\n", (long long)n, total_ms / repeats, repeats);
+    hipFree(d_a); hipFree(d_z); hipFree(d_w);
+    return 0;
+  }
   HIP_OK(hipMemcpy(z.data(), d_z, z.size() * sizeof(double), hipMemcpyDeviceToHost));
   HIP_OK(hipMemcpy(w.data(), d_w, w.size() * sizeof(double), hipMemcpyDeviceToHost));
   double worst_res = 0.0, worst_orth = 0.0, scale = 0.0;
@@ -119,14 +163,15 @@ static int check_eigh(int64_t n) {
 }
 
 int main(int argc, char** argv) {
-  if (argc == 3 && std::string(argv[1]) == "qr") return check_qr(std::atoll(argv[2]));
-  if (argc == 3 && std::string(argv[1]) == "eigh") return check_eigh(std::atoll(argv[2]));
+  const bool timed_only = argc == 4 && std::string(argv[3]) == "timed";
+  if ((argc == 3 || timed_only) && std::string(argv[1]) == "qr") return check_qr(std::atoll(argv[2]), timed_only);
+  if ((argc == 3 || timed_only) && std::string(argv[1]) == "eigh") return check_eigh(std::atoll(argv[2]), timed_only);
   const int64_t rows = argc > 2 ? std::atoll(argv[1]) : 4096;
   const int64_t cols = argc > 2 ? std::atoll(argv[2]) : 11008;
   const int repeats = argc > 3 ? std::atoi(argv[3]) : 5;
   const int copies = argc > 4 ? std::atoi(argv[4]) : 3;
   if (rows <= 0 || cols <= 0 || repeats <= 0 || copies < 0) {
-    std::fprintf(stderr, "usage: abi_probe [rows cols [repeats [copies]]]\n");
+    std::fprintf(stderr, "usage: abi_probe [rows cols [repeats [copies]]]  | abi_probe qr N [timed]  | abi_probe eigh N [timed]\n");
     return 1;
   }
   std::printf("backend %s, %lld x %lld, %d calls, %d calibration copies\n", soapmi_compiled_gpu_backend(),

@@ -308,3 +308,34 @@ def test_refresh_bases_and_transport_optimizer_state(shape, storage, device):
         if storage == "lower":  # the refresh rebuilt the upper triangle from the lower one
             p = dev[f"{side}_preconditioner"]
             assert torch.equal(p, p.T)
+
+
+def test_refresh_on_one_stream_gives_the_same_bits(device):
+    """`refresh_streams` only changes where the two factorisation chains are enqueued."""
+    from soap_tp_amd import _native
+    rows, columns = 300, 520
+    results = []
+    try:
+        for streams in (2, 1):
+            _native.call("soapmi_set_option", b"refresh_streams", streams)
+            dev = {
+                "momentum": column_major(make_matrix(rows, columns, seed=SEED + 3000), device),
+                "variance": column_major(make_matrix(rows, columns, seed=SEED + 4000).square(), device),
+                "left_preconditioner": column_major(make_preconditioner(rows, SEED + 5000), device),
+                "right_preconditioner": column_major(make_preconditioner(columns, SEED + 6000), device),
+                "left_basis": column_major(make_orthogonal(rows, SEED + 7000), device),
+                "right_basis": column_major(make_orthogonal(columns, SEED + 8000), device),
+            }
+            left_work = ops.allocate_2d_block_cyclic((rows, rows), BLOCK, GRID, device=device)
+            right_work = ops.allocate_2d_block_cyclic((columns, columns), BLOCK, GRID, device=device)
+            orders = ops.refresh_bases_and_transport_optimizer_state_(
+                dev["momentum"], dev["variance"], dev["left_preconditioner"], dev["right_preconditioner"],
+                dev["left_basis"], dev["right_basis"], left_work, right_work, (rows, columns), BLOCK, GRID)
+            results.append(([o.tolist() for o in orders], {name: t.cpu() for name, t in dev.items()}))
+    finally:
+        _native.call("soapmi_set_option", b"refresh_streams", 2)
+    assert results[0][0] == results[1][0]
+    for name in results[0][1]:
+        assert torch.equal(results[0][1][name], results[1][1][name]), name
+    with pytest.raises(ValueError):
+        _native.call("soapmi_set_option", b"refresh_streams", 3)
