@@ -230,12 +230,12 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
       }
       vi = Vc[r + (int64_t)i * ldw];
       T y = T(0);
-      for (int c0 = 0; c0 < n_slots; c0 += 16) {  // 16 slot loads in flight, summed in slot order
-        T yp[16];
+      for (int c0 = 0; c0 < n_slots; c0 += 32) {  // 32 slot loads in flight, summed in slot order
+        T yp[32];
 #pragma unroll
-        for (int c = 0; c < 16; ++c) yp[c] = (c0 + c < n_slots) ? y_part[(int64_t)(c0 + c) * n + r] : T(0);
+        for (int c = 0; c < 32; ++c) yp[c] = (c0 + c < n_slots) ? y_part[(int64_t)(c0 + c) * n + r] : T(0);
 #pragma unroll
-        for (int c = 0; c < 16; ++c) y += yp[c];
+        for (int c = 0; c < 32; ++c) y += yp[c];
       }
       T corr = T(0);
 #pragma unroll
