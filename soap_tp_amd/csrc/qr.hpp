@@ -4,7 +4,7 @@
 //
 // Panel (NB = 32 columns): a workgroup owns 256 rows, one per thread, and keeps its row of the
 // panel in registers.  Normally the whole panel runs in one persistent launch whose workgroups
-// exchange partial dot products through device memory, two columns per exchange
+// exchange partial dot products through device memory, up to four columns per exchange
 // (qr_panel_persistent_kernel); beyond kQrPersistentMaxWg workgroups it runs one launch per column
 // (qr_panel_step_kernel: launch j applies reflector j, whose dot products with the remaining
 // panel columns were reduced by launch j-1, and in the same pass reduces the dot products reflector
