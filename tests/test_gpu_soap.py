@@ -278,3 +278,25 @@ def test_properties_at_benchmark_sizes(shape, rank, device):
     assert abs(state["momentum"].double().norm().item() / momentum_norm - 1) <= 1e-4
     assert torch.equal(torch.sort(left_order).values, torch.arange(rows, device=device))
     assert torch.equal(torch.sort(right_order).values, torch.arange(columns, device=device))
+
+
+@pytest.mark.parametrize("scale", [0.0, 1e-20, 1e8])
+@pytest.mark.parametrize("shape", [(96, 160), (300, 200)])
+def test_extreme_gradient_magnitudes_stay_finite(scale, shape, device):
+    """All-zero gradients, gradients whose squares underflow and very large ones: every update stays
+    finite and the bases stay orthogonal through initialisation and two refreshes (the Gram matrices
+    are then zero, flushed to zero, or of the order of 1e19)."""
+    rows, columns = shape
+    generator = torch.Generator().manual_seed(SEED + 77)
+    state = {}
+    for _ in range(8):
+        gradient = (torch.randn(rows, columns, generator=generator) * scale).to(device)
+        update = soap_tp_amd.soap_step(gradient, state, global_shape=shape, shard_dim=1, block_size=128,
+                                       process_grid_shape=(1, 1), basis_refresh_interval=3)
+        assert torch.isfinite(update).all()
+        if scale == 0.0:
+            assert not update.any()
+    for side, size in (("left", rows), ("right", columns)):
+        basis = state[f"{side}_basis"]
+        assert torch.isfinite(basis).all()
+        torch.testing.assert_close(basis.T @ basis, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
