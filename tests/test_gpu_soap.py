@@ -300,3 +300,21 @@ def test_extreme_gradient_magnitudes_stay_finite(scale, shape, device):
         basis = state[f"{side}_basis"]
         assert torch.isfinite(basis).all()
         torch.testing.assert_close(basis.T @ basis, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
+
+
+def test_nan_gradient_propagates_without_hanging(device):
+    """A NaN in one gradient poisons the updates from that step on (as it does in the reference's
+    arithmetic) and every kernel still terminates: the factorisations' bounded waits and iteration
+    caps hold for non-finite data, through two refreshes."""
+    shape = (96, 160)
+    generator = torch.Generator().manual_seed(SEED + 78)
+    state = {}
+    seen = []
+    for step in range(6):
+        gradient = torch.randn(*shape, generator=generator) * 1e-2
+        if step == 2:
+            gradient[3, 5] = float("nan")
+        update = soap_tp_amd.soap_step(gradient.to(device), state, global_shape=shape, shard_dim=1, block_size=128,
+                                       process_grid_shape=(1, 1), basis_refresh_interval=2)
+        seen.append(bool(torch.isnan(update).any()))
+    assert seen == [False, False, True, True, True, True]
