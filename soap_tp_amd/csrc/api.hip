@@ -435,18 +435,13 @@ int soapmi_argsort_desc_f32(const float* keys, int64_t n, int64_t* order, void* 
   return kOk;
 }
 
-static inline dim3 grid_rows_cols(int64_t rows, int64_t cols) {
-  return dim3((unsigned)ceil_div64(rows, 256), (unsigned)(cols < 8192 ? (cols > 0 ? cols : 1) : 8192));
-}
-
 int soapmi_gather_f32(const float* in, int64_t ldi, float* out, int64_t ldo, int64_t rows, int64_t cols,
                       const int64_t* row_order, const int64_t* col_order, void* stream) {
   SOAPMI_REQUIRE(rows >= 0 && cols >= 0, "matrix dimensions must be non-negative");
   if (rows == 0 || cols == 0) return kOk;
   SOAPMI_REQUIRE(in && out && in != out, "buffers must be nonzero and distinct");
   SOAPMI_REQUIRE(ldi >= rows && ldo >= rows, "leading dimensions are too small");
-  hipLaunchKernelGGL((gather2d_kernel<float>), grid_rows_cols(rows, cols), dim3(256), 0, (hipStream_t)stream, in, ldi,
-                     out, ldo, (int)rows, (int)cols, row_order, col_order);
+  launch_gather2d((hipStream_t)stream, in, ldi, out, ldo, rows, cols, row_order, col_order);
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
@@ -459,10 +454,8 @@ size_t soapmi_permute_workspace_bytes(int64_t rows, int64_t cols) {
 
 static int permute_with(hipStream_t s, float* matrix, int64_t ld, int64_t rows, int64_t cols,
                         const int64_t* row_order, const int64_t* col_order, float* tmp) {
-  hipLaunchKernelGGL((gather2d_kernel<float>), grid_rows_cols(rows, cols), dim3(256), 0, s, matrix, ld, tmp, rows,
-                     (int)rows, (int)cols, row_order, col_order);
-  hipLaunchKernelGGL((copy2d_kernel<float>), grid_rows_cols(rows, cols), dim3(256), 0, s, tmp, rows, matrix, ld,
-                     (int)rows, (int)cols);
+  launch_gather2d(s, matrix, ld, tmp, rows, rows, cols, row_order, col_order);
+  launch_gather2d(s, tmp, rows, matrix, ld, rows, cols, nullptr, nullptr);  // copy back
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }

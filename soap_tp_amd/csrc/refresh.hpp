@@ -93,7 +93,13 @@ __global__ void argsort_finish_kernel(const int* id, int n, int64_t* order) {
 }
 
 // out[i, j] = in[row_order[i], col_order[j]]  (optimizer.py:408 semantics); a null order is the
-// identity.  Lanes run along i, so reads are coalesced whenever rows are not permuted.
+// identity.  Three kernels, chosen by launch_gather2d:
+//   gather2d_columns_kernel  rows not permuted, everything 16-byte aligned: a thread moves four
+//                            consecutive rows of a column per load, eight columns per thread
+//   gather2d_lds_kernel      rows permuted, a source column fits in LDS: a workgroup reads two source
+//                            columns with coalesced loads, then serves its output rows from LDS, so
+//                            the matrix crosses HBM once each way however scattered the row order is
+//   gather2d_kernel          anything else (lanes along i: coalesced when rows are not permuted)
 template <typename T>
 __global__ void gather2d_kernel(const T* __restrict__ in, int64_t ldi, T* __restrict__ out, int64_t ldo, int rows,
                                 int cols, const int64_t* __restrict__ row_order,
@@ -107,12 +113,76 @@ __global__ void gather2d_kernel(const T* __restrict__ in, int64_t ldi, T* __rest
   }
 }
 
+constexpr int kGatherColsPerThread = 8;
+
+__global__ __launch_bounds__(256) void gather2d_columns_kernel(const float* __restrict__ in, int64_t ldi,
+                                                               float* __restrict__ out, int64_t ldo, int rows, int cols,
+                                                               const int64_t* __restrict__ col_order) {
+  const int i4 = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i4 >= rows) return;
+  const int j0 = blockIdx.y * kGatherColsPerThread;
+  float4 v[kGatherColsPerThread];
+#pragma unroll
+  for (int c = 0; c < kGatherColsPerThread; ++c) {
+    const int j = min(j0 + c, cols - 1);
+    const int64_t sj = col_order ? col_order[j] : (int64_t)j;
+    v[c] = *reinterpret_cast<const float4*>(in + i4 + sj * ldi);
+  }
+#pragma unroll
+  for (int c = 0; c < kGatherColsPerThread; ++c)
+    if (j0 + c < cols) *reinterpret_cast<float4*>(out + i4 + (int64_t)(j0 + c) * ldo) = v[c];
+}
+
+constexpr int kGatherLdsRows = 8192;  // two source columns of this many floats: 64 KB of LDS
+
+__global__ __launch_bounds__(256) void gather2d_lds_kernel(const float* __restrict__ in, int64_t ldi,
+                                                           float* __restrict__ out, int64_t ldo, int rows, int cols,
+                                                           const int64_t* __restrict__ row_order,
+                                                           const int64_t* __restrict__ col_order) {
+  __shared__ float column[2][kGatherLdsRows];
+  const int j0 = 2 * blockIdx.x;
+  const bool second = j0 + 1 < cols;
+  const int64_t s0 = col_order ? col_order[j0] : (int64_t)j0;
+  const int64_t s1 = second ? (col_order ? col_order[j0 + 1] : (int64_t)(j0 + 1)) : s0;
+  for (int i = threadIdx.x; i < rows; i += 256) {
+    column[0][i] = in[i + s0 * ldi];
+    column[1][i] = in[i + s1 * ldi];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < rows; i += 256) {
+    const int si = (int)row_order[i];
+    out[i + (int64_t)j0 * ldo] = column[0][si];
+    if (second) out[i + (int64_t)(j0 + 1) * ldo] = column[1][si];
+  }
+}
+
 template <typename T>
 __global__ void copy2d_kernel(const T* __restrict__ in, int64_t ldi, T* __restrict__ out, int64_t ldo, int rows,
                               int cols) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= rows) return;
   for (int j = blockIdx.y; j < cols; j += gridDim.y) out[i + (int64_t)j * ldo] = in[i + (int64_t)j * ldi];
+}
+
+static inline bool aligned16_columns(const void* p, int64_t ld, int64_t rows) {
+  return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0 && rows % 4 == 0;
+}
+
+// out = in[row_order][:, col_order] (null orders: identity) with the kernel that fits.
+static inline void launch_gather2d(hipStream_t s, const float* in, int64_t ldi, float* out, int64_t ldo, int64_t rows,
+                                   int64_t cols, const int64_t* row_order, const int64_t* col_order) {
+  if (rows <= 0 || cols <= 0) return;
+  if (!row_order && aligned16_columns(in, ldi, rows) && aligned16_columns(out, ldo, rows)) {
+    const dim3 grid((unsigned)ceil_div64(rows, 1024), (unsigned)ceil_div64(cols, kGatherColsPerThread));
+    hipLaunchKernelGGL(gather2d_columns_kernel, grid, dim3(256), 0, s, in, ldi, out, ldo, (int)rows, (int)cols, col_order);
+  } else if (row_order && rows <= kGatherLdsRows) {
+    hipLaunchKernelGGL(gather2d_lds_kernel, dim3((unsigned)ceil_div64(cols, 2)), dim3(256), 0, s, in, ldi, out, ldo,
+                       (int)rows, (int)cols, row_order, col_order);
+  } else {
+    const dim3 grid((unsigned)ceil_div64(rows, 256), (unsigned)(cols < 8192 ? cols : 8192));
+    hipLaunchKernelGGL((gather2d_kernel<float>), grid, dim3(256), 0, s, in, ldi, out, ldo, (int)rows, (int)cols,
+                       row_order, col_order);
+  }
 }
 
 // flags[0] = 1 unless `order` is a permutation of range(n).  `seen` must be zeroed (n ints).
