@@ -36,6 +36,7 @@ struct GemmProblem {
   int num_tiles;
   int lower;           // enumerate only tiles with tile_m >= tile_n (square tile grid)
   int k_chunk;         // K extent handled by one blockIdx.y slice (multiple of BK)
+  const int* ksel_b;   // general path, B operand x-contiguous only: row k of op(B) is stored as row ksel_b[k] (null: k)
 };
 
 // ---- epilogues ---------------------------------------------------------------------------
@@ -146,7 +147,8 @@ __device__ __forceinline__ int kcontig_kv(int v) {
 // xcontig: element (x, k) lives at base[x + k*ld]; otherwise at base[k + x*ld].
 template <typename T, int BX, int BK, int NT, int NV>
 __device__ __forceinline__ void load_slab(T (&reg)[NV][Vec16<T>::W], const T* __restrict__ base, int64_t ld,
-                                          int x0, int X, int k0, int kend, bool xcontig, bool vec, int tid) {
+                                          int x0, int X, int k0, int kend, bool xcontig, bool vec, int tid,
+                                          const int* __restrict__ ksel = nullptr) {
   constexpr int VW = Vec16<T>::W;
   using V = typename Vec16<T>::type;
 #pragma unroll
@@ -155,7 +157,8 @@ __device__ __forceinline__ void load_slab(T (&reg)[NV][Vec16<T>::W], const T* __
     if (xcontig) {
       int k = v / (BX / VW), xv = v % (BX / VW);
       int gx = x0 + xv * VW, gk = k0 + k;
-      const T* p = base + gx + (int64_t)gk * ld;
+      const int64_t sk = (ksel && gk < kend) ? ksel[gk] : gk;  // stored row of this k
+      const T* p = base + gx + sk * ld;
       if (vec) {
         if (gx < X && gk < kend) {
           V t = *reinterpret_cast<const V*>(p);
@@ -317,7 +320,7 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
       fb.load(rb);
     } else {
       load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, kbeg, kend, a_xc, p.vecA, tid);
-      load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, kbeg, kend, b_xc, p.vecB, tid);
+      load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, kbeg, kend, b_xc, p.vecB, tid, p.ksel_b);
     }
     store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[0], ra, a_xc, tid);
     store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[0], rb, b_xc, tid);
@@ -334,7 +337,7 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
       } else {
         const int k0 = kbeg + (kt + 1) * BK;
         load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, k0, kend, a_xc, p.vecA, tid);
-        load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, k0, kend, b_xc, p.vecB, tid);
+        load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, k0, kend, b_xc, p.vecB, tid, p.ksel_b);
       }
     }
     const T* as = As[buf];
@@ -418,6 +421,7 @@ __device__ __forceinline__ void fill_batched(BatchedGemm<T>& b, int transA, int 
   b.p.tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
   b.p.num_tiles = b.p.tiles_m * b.p.tiles_n;
   b.p.lower = 0;
+  b.p.ksel_b = nullptr;
   b.p.k_chunk = ((K > 0 ? K : 1) + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
   b.e.C = C; b.e.ldc = ldc; b.e.alpha = alpha; b.e.beta = beta;
 }
@@ -500,6 +504,7 @@ static inline GemmProblem<T> make_problem(int transA, int transB, int M, int N, 
   p.tiles_m = (int)ceil_div64(M, Cfg::BM);
   p.tiles_n = (int)ceil_div64(N, Cfg::BN);
   p.lower = lower ? 1 : 0;
+  p.ksel_b = nullptr;
   p.num_tiles = lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
   p.k_chunk = (int)(ceil_div64(K > 0 ? K : 1, Cfg::BK) * Cfg::BK);
   return p;

@@ -14,7 +14,13 @@
 // eigenvector columns; solve the secular equation with a bracketed rational ("middle way")
 // iteration that falls back to bisection, one thread per root in small merges and one wavefront
 // per root (poles spread over the lanes) in merges of 256 and more; recompute the update vector
-// from the roots; form the k x k eigenvector matrix of the rank-one update; multiply (MFMA).
+// from the roots; form the k x k eigenvector matrix of the rank-one update; multiply (MFMA).  The
+// children's eigenvectors are block diagonal, so a surviving column has support in the top rows,
+// the bottom rows, or (after a deflation rotation across the children) both: the deflation scan
+// records which, the gather packs the top-supported columns for the top rows and the
+// bottom-supported ones for the bottom rows, and the product is done as two half-height products
+// whose B operand picks the matching rows of the rank-one eigenvector matrix (about half the flops
+// of multiplying the zero blocks along).
 // Eigenvector columns are not kept in sorted order between levels (the sort permutation is
 // recomputed where it is needed); one final sort orders the result.
 #pragma once
@@ -46,7 +52,13 @@ struct DcWorkspace {
   int* rot_b;  // n
   int* kcount; // n   per merge: k, or -1 for a merge with an empty child
   int* nrot;   // n
-  BatchedGemm<T>* batch;  // n
+  int* pos1;   // n   per non-deflated pole: its column among the top-supported ones, or -1
+  int* pos2;   // n   the same for the bottom rows
+  int* sel1;   // n   per merge, compact at [lo, lo+k1): the poles with support in the top rows
+  int* sel2;   // n   the same for the bottom rows
+  int* kc1;    // n   per merge: number of top-supported poles
+  int* kc2;    // n
+  BatchedGemm<T>* batch;  // 2n: two products per merge
   T* X;  // n x n eigenvectors (block diagonal by level)
   T* S;  // n x n secular differences / rank-one eigenvectors
   int64_t ldx, lds;
@@ -74,7 +86,13 @@ static inline void dc_workspace_layout(WS& ws, int64_t n, DcWorkspace<T>* out) {
   w.rot_b = ws.template take<int>(n);
   w.kcount = ws.template take<int>(n);
   w.nrot = ws.template take<int>(n);
-  w.batch = ws.template take<BatchedGemm<T>>(n);
+  w.pos1 = ws.template take<int>(n);
+  w.pos2 = ws.template take<int>(n);
+  w.sel1 = ws.template take<int>(n);
+  w.sel2 = ws.template take<int>(n);
+  w.kc1 = ws.template take<int>(n);
+  w.kc2 = ws.template take<int>(n);
+  w.batch = ws.template take<BatchedGemm<T>>(2 * n);
   w.X = ws.template take<T>((size_t)n * n);
   w.S = ws.template take<T>((size_t)n * n);
   w.ldx = n;
@@ -195,7 +213,10 @@ __global__ __launch_bounds__(256) void dc_deflate_kernel(int t, int n, int np, T
                                                          int* __restrict__ idx, int* __restrict__ rot_a,
                                                          int* __restrict__ rot_b, T* __restrict__ rot_c,
                                                          T* __restrict__ rot_s, int* __restrict__ kcount,
-                                                         int* __restrict__ nrot_out) {
+                                                         int* __restrict__ nrot_out, int* __restrict__ pos1,
+                                                         int* __restrict__ pos2, int* __restrict__ sel1,
+                                                         int* __restrict__ sel2, int* __restrict__ kc1,
+                                                         int* __restrict__ kc2) {
   constexpr int CH = 1024;
   __shared__ T s_d[CH];
   __shared__ T s_z[CH];
@@ -205,10 +226,11 @@ __global__ __launch_bounds__(256) void dc_deflate_kernel(int t, int n, int np, T
   const int tid = threadIdx.x;
   const DcMerge m = dc_merge(t, q, n);
   if (m.empty()) {
-    if (tid == 0) { kcount[q] = -1; nrot_out[q] = 0; }
+    if (tid == 0) { kcount[q] = -1; nrot_out[q] = 0; kc1[q] = 0; kc2[q] = 0; }
     return;
   }
   const int lo = m.lo, N = m.hi - m.lo;
+  const int n_top = m.mid - m.lo;  // columns [0, n_top) of the block belong to the first child
   const T rho = T(2) * fabs(e[m.mid - 1]);
   T dm = T(0), zm = T(0);
   for (int c = tid; c < N; c += 256) {
@@ -229,11 +251,20 @@ __global__ __launch_bounds__(256) void dc_deflate_kernel(int t, int n, int np, T
   const T tol = T(8) * eps * fmax(dm, zm);
   if (rho * zm <= tol) {  // nothing couples: the children's eigenpairs are the parent's
     for (int c = tid; c < N; c += 256) { idx[lo + c] = c; dnew[lo + c] = d[lo + c]; }
-    if (tid == 0) { kcount[q] = 0; nrot_out[q] = 0; }
+    if (tid == 0) { kcount[q] = 0; nrot_out[q] = 0; kc1[q] = 0; kc2[q] = 0; }
     return;
   }
   int pj = -1, k = 0, ndefl = 0, nrot = 0;
+  int sup_pj = 0, c1 = 0, c2 = 0;  // support of the candidate column: bit 0 top rows, bit 1 bottom rows
   T d_pj = T(0), z_pj = T(0);
+  auto keep = [&](int col, T dval, T zval, int sup) {  // a pole of the secular equation
+    idx[lo + k] = col; dl[lo + k] = dval; wv[lo + k] = zval;
+    pos1[lo + k] = (sup & 1) ? c1 : -1;
+    pos2[lo + k] = (sup & 2) ? c2 : -1;
+    if (sup & 1) sel1[lo + c1++] = k;
+    if (sup & 2) sel2[lo + c2++] = k;
+    ++k;
+  };
   const int64_t sbase = (int64_t)q * np;
   for (int base = 0; base < N; base += CH) {
     const int cnt = min(CH, N - base);
@@ -255,7 +286,9 @@ __global__ __launch_bounds__(256) void dc_deflate_kernel(int t, int n, int np, T
           dnew[lo + slot] = dj;
         } else if (pj < 0) {
           pj = nj; d_pj = dj; z_pj = zj;
+          sup_pj = nj < n_top ? 1 : 2;
         } else {
+          const int sup_nj = nj < n_top ? 1 : 2;
           T ss = z_pj, cc = zj;
           const T tau = hypot(cc, ss);
           const T tt = dj - d_pj;
@@ -272,22 +305,22 @@ __global__ __launch_bounds__(256) void dc_deflate_kernel(int t, int n, int np, T
             idx[lo + slot] = pj;
             dnew[lo + slot] = t2;
             pj = nj; d_pj = dj; z_pj = zj;
+            sup_pj |= sup_nj;  // the rotation mixed the two columns
           } else {
-            idx[lo + k] = pj; dl[lo + k] = d_pj; wv[lo + k] = z_pj;
-            ++k;
+            keep(pj, d_pj, z_pj, sup_pj);
             pj = nj; d_pj = dj; z_pj = zj;
+            sup_pj = sup_nj;
           }
         }
       }
     }
   }
   if (tid == 0) {
-    if (pj >= 0) {
-      idx[lo + k] = pj; dl[lo + k] = d_pj; wv[lo + k] = z_pj;
-      ++k;
-    }
+    if (pj >= 0) keep(pj, d_pj, z_pj, sup_pj);
     kcount[q] = k;
     nrot_out[q] = nrot;
+    kc1[q] = c1;
+    kc2[q] = c2;
   }
 }
 
@@ -313,18 +346,25 @@ __global__ void dc_rotate_kernel(int t, int n, T* __restrict__ X, int64_t ldx, c
   }
 }
 
-// Y[:, s] = X[:, idx[s]] within the merged block (non-deflated columns first).
+// Within the merged block: deflated columns s >= k go to Y[:, s] = X[:, idx[s]]; a surviving column
+// s < k goes, for the top rows, to column pos1[s] (if it has support there) and, for the bottom
+// rows, to column pos2[s]: the two row ranges of Y hold two differently packed column sets.
 template <typename T>
 __global__ void dc_gather_kernel(int t, int n, const T* __restrict__ X, int64_t ldx, T* __restrict__ Y, int64_t ldy,
-                                 const int* __restrict__ idx, const int* __restrict__ kcount) {
+                                 const int* __restrict__ idx, const int* __restrict__ kcount,
+                                 const int* __restrict__ pos1, const int* __restrict__ pos2) {
   const int q = blockIdx.z;
-  if (kcount[q] < 0) return;
+  const int k = kcount[q];
+  if (k < 0) return;
   const DcMerge m = dc_merge(t, q, n);
   const int r = m.lo + blockIdx.x * blockDim.x + threadIdx.x;
   if (r >= m.hi) return;
   const int N = m.hi - m.lo;
-  for (int s = blockIdx.y; s < N; s += gridDim.y)
-    Y[r + (int64_t)(m.lo + s) * ldy] = X[r + (int64_t)(m.lo + idx[m.lo + s]) * ldx];
+  const int* pos = (r < m.mid) ? pos1 : pos2;
+  for (int s = blockIdx.y; s < N; s += gridDim.y) {
+    const int dst = (s < k) ? pos[m.lo + s] : s;
+    if (dst >= 0) Y[r + (int64_t)(m.lo + dst) * ldy] = X[r + (int64_t)(m.lo + idx[m.lo + s]) * ldx];
+  }
 }
 
 // Root i of 1 + rho * sum_j w_j^2 / (dl_j - lambda) = 0 on (dl_i, dl_{i+1}).  The unknown is the
@@ -598,8 +638,10 @@ __global__ void dc_form_u_kernel(int t, int n, const int* __restrict__ kcount, c
 }
 
 template <typename T>
-__global__ void dc_setup_gemm_kernel(int t, int n, int nq, const int* __restrict__ kcount, const T* __restrict__ Y,
-                                     int64_t ldy, const T* __restrict__ S, int64_t lds, T* __restrict__ X, int64_t ldx,
+__global__ void dc_setup_gemm_kernel(int t, int n, int nq, const int* __restrict__ kcount, const int* __restrict__ kc1,
+                                     const int* __restrict__ kc2, const int* __restrict__ sel1,
+                                     const int* __restrict__ sel2, const T* __restrict__ Y, int64_t ldy,
+                                     const T* __restrict__ S, int64_t lds, T* __restrict__ X, int64_t ldx,
                                      BatchedGemm<T>* __restrict__ batch) {
   using Cfg = typename DefaultTile<T>::type;
   const int q = blockIdx.x * blockDim.x + threadIdx.x;
@@ -608,15 +650,22 @@ __global__ void dc_setup_gemm_kernel(int t, int n, int nq, const int* __restrict
   BatchedGemm<T> b;
   if (k <= 0) {
     b.p.M = 0; b.p.N = 0; b.p.K = 0; b.p.num_tiles = 0;
-    batch[q] = b;
+    batch[2 * q] = b;
+    batch[2 * q + 1] = b;
     return;
   }
   const DcMerge m = dc_merge(t, q, n);
-  const int N = m.hi - m.lo;
   const int64_t o = m.lo;
-  // X[:, 0:k] = Y[:, 0:k] * U with U[j, i] = S[i + j*lds] (stored transposed)
-  fill_batched<T, Cfg>(b, 0, 1, N, k, k, Y + o + o * ldy, ldy, S + o + o * lds, lds, X + o + o * ldx, ldx, T(1), T(0));
-  batch[q] = b;
+  // X[rows, 0:k] = Y[rows, 0:k_half] * U[sel, :] with U[j, i] = S[i + j*lds] (stored transposed), once
+  // for the top rows with the top-supported poles and once for the bottom rows
+  fill_batched<T, Cfg>(b, 0, 1, m.mid - m.lo, k, kc1[q], Y + o + o * ldy, ldy, S + o + o * lds, lds, X + o + o * ldx, ldx,
+                       T(1), T(0));
+  b.p.ksel_b = sel1 + m.lo;
+  batch[2 * q] = b;
+  fill_batched<T, Cfg>(b, 0, 1, m.hi - m.mid, k, kc2[q], Y + m.mid + o * ldy, ldy, S + o + o * lds, lds,
+                       X + m.mid + o * ldx, ldx, T(1), T(0));
+  b.p.ksel_b = sel2 + m.lo;
+  batch[2 * q + 1] = b;
 }
 
 // Deflated columns pass through unchanged; d takes the merged eigenvalues.
@@ -696,11 +745,12 @@ static inline int stedc(hipStream_t s, int n, const T* d0, const T* e0, T* w_out
                        ws.ldx, ws.d, ws.e, ws.z, ws.skey, ws.sidx);
     dc_batched_sort<T>(s, ws, np, nq);
     hipLaunchKernelGGL((dc_deflate_kernel<T>), dim3(nq), dim3(256), 0, s, t, n, np, ws.d, ws.e, ws.z, ws.sidx, ws.dl,
-                       ws.wv, ws.dnew, ws.idx, ws.rot_a, ws.rot_b, ws.rot_c, ws.rot_s, ws.kcount, ws.nrot);
+                       ws.wv, ws.dnew, ws.idx, ws.rot_a, ws.rot_b, ws.rot_c, ws.rot_s, ws.kcount, ws.nrot, ws.pos1, ws.pos2,
+                       ws.sel1, ws.sel2, ws.kc1, ws.kc2);
     hipLaunchKernelGGL((dc_rotate_kernel<T>), dim3(rbl, nq), dim3(256), 0, s, t, n, ws.X, ws.ldx, ws.rot_a, ws.rot_b,
                        ws.rot_c, ws.rot_s, ws.nrot);
     hipLaunchKernelGGL((dc_gather_kernel<T>), dim3(rbl, ycols, nq), dim3(256), 0, s, t, n, ws.X, ws.ldx, Y, ldy, ws.idx,
-                       ws.kcount);
+                       ws.kcount, ws.pos1, ws.pos2);
     if (nmax >= 256) {
       hipLaunchKernelGGL((dc_secular_wave_kernel<T>), dim3((unsigned)ceil_div64(nmax, 4), nq), dim3(256), 0, s, t, n,
                          ws.e, ws.dl, ws.wv, ws.kcount, ws.dnew, ws.mu, ws.org);
@@ -714,10 +764,11 @@ static inline int stedc(hipStream_t s, int n, const T* d0, const T* e0, T* w_out
                        ws.zhat);
     hipLaunchKernelGGL((dc_form_u_kernel<T>), dim3(rbl, nq), dim3(256), 0, s, t, n, ws.kcount, ws.zhat, ws.S, ws.lds);
     hipLaunchKernelGGL((dc_setup_gemm_kernel<T>), dim3((unsigned)ceil_div64(nq, 256)), dim3(256), 0, s, t, n, nq,
-                       ws.kcount, Y, ldy, ws.S, ws.lds, ws.X, ws.ldx, ws.batch);
-    const int tiles = (int)(ceil_div64(nmax, Cfg::BM) * ceil_div64(nmax, Cfg::BN));
-    hipLaunchKernelGGL((gemm_batched_kernel<T, Cfg>), dim3(8 * (unsigned)ceil_div64(tiles, 8), 1, nq), dim3(Cfg::NT), 0,
-                       s, ws.batch);
+                       ws.kcount, ws.kc1, ws.kc2, ws.sel1, ws.sel2, Y, ldy, ws.S, ws.lds, ws.X, ws.ldx, ws.batch);
+    const int half = nmax / 2 + 1;  // a child has at most this many rows
+    const int tiles = (int)(ceil_div64(half, Cfg::BM) * ceil_div64(nmax, Cfg::BN));
+    hipLaunchKernelGGL((gemm_batched_kernel<T, Cfg>), dim3(8 * (unsigned)ceil_div64(tiles, 8), 1, 2 * nq), dim3(Cfg::NT),
+                       0, s, ws.batch);
     hipLaunchKernelGGL((dc_finish_kernel<T>), dim3(rbl, ycols, nq), dim3(256), 0, s, t, n, ws.kcount, Y, ldy, ws.X,
                        ws.ldx, ws.dnew, ws.d);
     SOAPMI_LAUNCH_CHECK();

@@ -134,6 +134,44 @@ def test_eigh_f64_c_abi_directly(device):
         _native.call("soapmi_eigh_f64", a.data_ptr(), w.data_ptr(), q.data_ptr(), size, size - 1, size, None, 0, None)
 
 
+@pytest.mark.parametrize("kind", ["clusters", "glued_wilkinson", "block_diagonal"])
+def test_eigh_f64_with_heavy_deflation(kind, device):
+    """Spectra that make the divide and conquer deflate: eigenvalues repeated in groups (rotations
+    between columns of the two children of a merge), glued Wilkinson blocks (pairs that agree to
+    working precision) and an exactly decoupled block-diagonal matrix (whole merges with nothing to
+    solve).  Checked through invariants: spectrum against LAPACK, orthogonality, residual."""
+    size = 520
+    generator = torch.Generator().manual_seed(SEED + 91)
+    if kind == "clusters":
+        basis, _ = torch.linalg.qr(torch.randn(size, size, generator=generator, dtype=torch.float64))
+        spectrum = torch.tensor([0.0, 1e-9, 0.5, 1.0, 1.0 + 1e-13, 2.0, 7.0, 7.5], dtype=torch.float64)
+        matrix = (basis * spectrum[torch.randint(0, len(spectrum), (size,), generator=generator)]) @ basis.T
+        matrix = (matrix + matrix.T) / 2
+    elif kind == "glued_wilkinson":
+        block = 21
+        w21 = torch.diag((torch.arange(block) - block // 2).abs().double()) + torch.diag(torch.ones(block - 1), 1).double() \
+            + torch.diag(torch.ones(block - 1), -1).double()
+        copies = size // block + 1
+        matrix = torch.block_diag(*[w21] * copies)[:size, :size].clone()
+        for c in range(1, copies):  # weak glue between neighbouring blocks
+            if c * block < size:
+                matrix[c * block, c * block - 1] = matrix[c * block - 1, c * block] = 1e-8
+    else:
+        g = torch.randn(size // 2, size // 2, generator=generator, dtype=torch.float64)
+        matrix = torch.block_diag(g + g.T, 3.0 * torch.eye(size - size // 2, dtype=torch.float64))
+    a = column_major(torch.tril(matrix), device)
+    q = torch.zeros(size, size, dtype=torch.float64, device=device).T
+    w = torch.zeros(size, dtype=torch.float64, device=device)
+    _native.call("soapmi_eigh_f64", a.data_ptr(), w.data_ptr(), q.data_ptr(), size, size, size, None, 0,
+                 torch.cuda.current_stream().cuda_stream)
+    expected = torch.linalg.eigvalsh(matrix)
+    scale = max(expected.abs().max().item(), 1.0)
+    assert torch.allclose(w.cpu(), expected, rtol=0, atol=1e-12 * scale * size)
+    qc = q.cpu()
+    assert (qc.T @ qc - torch.eye(size, dtype=torch.float64)).abs().max().item() < 1e-12
+    assert (matrix @ qc - qc * w.cpu()).abs().max().item() < 1e-11 * scale
+
+
 def test_injected_elpa_binding_follows_reference_staging(device):
     from soap_tp_amd.binding import NativeBinding
 
