@@ -40,6 +40,7 @@ struct DcWorkspace {
   T* wv;     // n   matching z components
   T* dnew;   // n
   T* zhat;   // n
+  T* norm_part;  // kDcNormChunks x n   partial squared norms of the rank-one eigenvectors
   T* mu;     // n   root offsets from their origin poles (wavefront-per-root path)
   int* org;  // n   origin pole of each root
   T* rot_c;  // n
@@ -74,6 +75,7 @@ static inline void dc_workspace_layout(WS& ws, int64_t n, DcWorkspace<T>* out) {
   w.wv = ws.template take<T>(n);
   w.dnew = ws.template take<T>(n);
   w.zhat = ws.template take<T>(n);
+  w.norm_part = ws.template take<T>((size_t)32 * n);
   w.mu = ws.template take<T>(n);
   w.org = ws.template take<int>(n);
   w.rot_c = ws.template take<T>(n);
@@ -618,23 +620,46 @@ __global__ __launch_bounds__(256) void dc_zhat_kernel(int t, int n, const T* __r
   }
 }
 
-// Column i of the rank-one eigenvector matrix, stored transposed in place of deltaT.
+// Column i of the rank-one eigenvector matrix, u_i[j] = zhat_j / deltaT[i, j] normalised, stored
+// transposed in place of deltaT.  Two passes over a 2-D grid (roots x kDcNormChunks slices of the
+// poles): partial squared norms, then every thread sums the partials of its root in slice order
+// and writes its slice.
+constexpr int kDcNormChunks = 32;
+
 template <typename T>
-__global__ void dc_form_u_kernel(int t, int n, const int* __restrict__ kcount, const T* __restrict__ zhat,
-                                 T* __restrict__ S, int64_t lds) {
-  const int q = blockIdx.y;
+__global__ void dc_form_u_norm_kernel(int t, int n, const int* __restrict__ kcount, const T* __restrict__ zhat,
+                                      const T* __restrict__ S, int64_t lds, T* __restrict__ norm_part) {
+  const int q = blockIdx.z;
   const int k = kcount[q];
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= k) return;
   const int lo = dc_bound(t, q, n);
-  T* row = S + (lo + i) + (int64_t)lo * lds;
+  const int chunk = (k + kDcNormChunks - 1) / kDcNormChunks;
+  const int j0 = blockIdx.y * chunk, j1 = min(k, j0 + chunk);
+  const T* row = S + (lo + i) + (int64_t)lo * lds;
   T nrm2 = T(0);
-  for (int j = 0; j < k; ++j) {
+  for (int j = j0; j < j1; ++j) {
     const T s = zhat[lo + j] / row[(int64_t)j * lds];
     nrm2 += s * s;
   }
+  norm_part[(int64_t)blockIdx.y * n + lo + i] = nrm2;
+}
+
+template <typename T>
+__global__ void dc_form_u_kernel(int t, int n, const int* __restrict__ kcount, const T* __restrict__ zhat,
+                                 T* __restrict__ S, int64_t lds, const T* __restrict__ norm_part) {
+  const int q = blockIdx.z;
+  const int k = kcount[q];
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= k) return;
+  const int lo = dc_bound(t, q, n);
+  const int chunk = (k + kDcNormChunks - 1) / kDcNormChunks;
+  const int j0 = blockIdx.y * chunk, j1 = min(k, j0 + chunk);
+  T nrm2 = T(0);
+  for (int c = 0; c < kDcNormChunks; ++c) nrm2 += norm_part[(int64_t)c * n + lo + i];
   const T inv = T(1) / sqrt(nrm2);
-  for (int j = 0; j < k; ++j) row[(int64_t)j * lds] = zhat[lo + j] / row[(int64_t)j * lds] * inv;
+  T* row = S + (lo + i) + (int64_t)lo * lds;
+  for (int j = j0; j < j1; ++j) row[(int64_t)j * lds] = zhat[lo + j] / row[(int64_t)j * lds] * inv;
 }
 
 template <typename T>
@@ -762,7 +787,10 @@ static inline int stedc(hipStream_t s, int n, const T* d0, const T* e0, T* w_out
     }
     hipLaunchKernelGGL((dc_zhat_kernel<T>), dim3(nmax, nq), dim3(256), 0, s, t, n, ws.dl, ws.wv, ws.kcount, ws.S, ws.lds,
                        ws.zhat);
-    hipLaunchKernelGGL((dc_form_u_kernel<T>), dim3(rbl, nq), dim3(256), 0, s, t, n, ws.kcount, ws.zhat, ws.S, ws.lds);
+    hipLaunchKernelGGL((dc_form_u_norm_kernel<T>), dim3(rbl, kDcNormChunks, nq), dim3(256), 0, s, t, n, ws.kcount, ws.zhat,
+                       ws.S, ws.lds, ws.norm_part);
+    hipLaunchKernelGGL((dc_form_u_kernel<T>), dim3(rbl, kDcNormChunks, nq), dim3(256), 0, s, t, n, ws.kcount, ws.zhat,
+                       ws.S, ws.lds, ws.norm_part);
     hipLaunchKernelGGL((dc_setup_gemm_kernel<T>), dim3((unsigned)ceil_div64(nq, 256)), dim3(256), 0, s, t, n, nq,
                        ws.kcount, ws.kc1, ws.kc2, ws.sel1, ws.sel2, Y, ldy, ws.S, ws.lds, ws.X, ws.ldx, ws.batch);
     const int half = nmax / 2 + 1;  // a child has at most this many rows
