@@ -386,12 +386,11 @@ static int next_pow2(int64_t n) {
   while (p < n) p <<= 1;
   return p;
 }
-constexpr int kArgsortLdsMax = 16384;
 
 size_t soapmi_argsort_workspace_bytes(int64_t n) {
   const int np2 = next_pow2(n);
   WorkspaceSizer w;
-  if (np2 > kArgsortLdsMax) {
+  if (n > kArgsortRankMax) {  // the global-memory bitonic network
     w.take<float>((size_t)np2);
     w.take<int>((size_t)np2);
   }
@@ -405,16 +404,9 @@ int soapmi_argsort_desc_f32(const float* keys, int64_t n, int64_t* order, void* 
   SOAPMI_REQUIRE(keys && order, "buffer addresses must be nonzero");
   hipStream_t s = (hipStream_t)stream;
   const int np2 = next_pow2(n);
-  if (np2 <= kArgsortLdsMax) {
-    const size_t lds = (size_t)np2 * (sizeof(float) + sizeof(int));
-    static bool attribute_set = false;
-    if (!attribute_set) {
-      SOAPMI_HIP(hipFuncSetAttribute((const void*)argsort_desc_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     kArgsortLdsMax * 8));
-      attribute_set = true;
-    }
-    const int threads = np2 >= 2048 ? 1024 : (np2 >= 128 ? np2 / 2 : 64);
-    hipLaunchKernelGGL(argsort_desc_lds_kernel, dim3(1), dim3(threads), lds, s, keys, (int)n, np2, order);
+  if (n <= kArgsortRankMax) {
+    const size_t lds = (size_t)((n + 3) & ~(int64_t)3) * sizeof(unsigned);  // all keys, at most 64 KB
+    hipLaunchKernelGGL(argsort_desc_rank_kernel, dim3((unsigned)ceil_div64(n, 64)), dim3(256), lds, s, keys, (int)n, order);
     SOAPMI_LAUNCH_CHECK();
     return kOk;
   }

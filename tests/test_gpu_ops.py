@@ -268,6 +268,13 @@ def test_argsort_ties_and_large(device):
         _native.call("soapmi_argsort_desc_f32", keys_dev.data_ptr(), count, order.data_ptr(), work.data_ptr(),
                      work.numel(), torch.cuda.current_stream().cuda_stream)
         assert order.tolist() == torch.argsort(keys, descending=True, stable=True).tolist()
+    # signed zeros tie, infinities order like numbers, NaNs go last in index order
+    special = torch.tensor([0.0, float("nan"), -0.0, float("inf"), -1.0, float("-inf"), 0.0, float("nan"), 2.5, -0.0])
+    order = torch.empty(special.numel(), dtype=torch.int64, device=device)
+    special_dev = special.to(device)
+    _native.call("soapmi_argsort_desc_f32", special_dev.data_ptr(), special.numel(), order.data_ptr(), None, 0,
+                 torch.cuda.current_stream().cuda_stream)
+    assert order.tolist() == [3, 8, 0, 2, 6, 9, 4, 5, 1, 7]
 
 
 # ---- refresh (tests/unit/test_factorizations.py:501-613) -----------------------------------------
