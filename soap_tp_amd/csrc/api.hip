@@ -375,8 +375,9 @@ int soapmi_column_dots_f32(const float* q, int64_t ldq, const float* work, int64
   if (cols == 0) return kOk;
   SOAPMI_REQUIRE(q && work && estimates, "buffer addresses must be nonzero");
   SOAPMI_REQUIRE(ldq >= rows && ldw >= rows, "leading dimensions are too small");
-  hipLaunchKernelGGL((coldot_kernel<float>), dim3((unsigned)cols), dim3(256), 0, (hipStream_t)stream, q, ldq, work, ldw,
-                     (int)rows, estimates);
+  const int vectors = aligned16_columns(q, ldq, rows) && aligned16_columns(work, ldw, rows) ? 1 : 0;
+  hipLaunchKernelGGL((coldot_kernel<float>), dim3((unsigned)ceil_div64(cols, 4)), dim3(256), 0, (hipStream_t)stream, q, ldq,
+                     work, ldw, (int)rows, (int)cols, estimates, vectors);
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }

@@ -5,22 +5,37 @@
 
 namespace soapmi {
 
-// est[j] = sum_i Q[i, j] * W[i, j]   (factorizations.py:255-257).  One workgroup per column,
-// fixed reduction tree, so the estimates (and hence the sort order) are reproducible.
+// est[j] = sum_i Q[i, j] * W[i, j]   (factorizations.py:255-257).  One wavefront per column (four
+// columns per workgroup); a lane takes every 64th group of four rows with 16-byte loads when the
+// columns are aligned for them, and the wavefront's partial sums meet in a fixed xor-butterfly: the
+// estimates, and hence the sort order, are reproducible.
 template <typename T>
-__global__ void coldot_kernel(const T* __restrict__ Q, int64_t ldq, const T* __restrict__ W, int64_t ldw, int n_rows,
-                              T* __restrict__ est) {
-  __shared__ T red[256];
-  const int j = blockIdx.x;
+__global__ __launch_bounds__(256) void coldot_kernel(const T* __restrict__ Q, int64_t ldq, const T* __restrict__ W,
+                                                     int64_t ldw, int n_rows, int n_cols, T* __restrict__ est,
+                                                     int vectors) {
+  const int lane = threadIdx.x & 63;
+  const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (j >= n_cols) return;
+  const T* q = Q + (int64_t)j * ldq;
+  const T* w = W + (int64_t)j * ldw;
   T s = T(0);
-  for (int i = threadIdx.x; i < n_rows; i += 256) s += Q[i + (int64_t)j * ldq] * W[i + (int64_t)j * ldw];
-  red[threadIdx.x] = s;
-  __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
-    if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
-    __syncthreads();
+  if (vectors) {
+    using V = typename Vec16<T>::type;
+    constexpr int VW = Vec16<T>::W;
+    for (int i = lane * VW; i < n_rows; i += 64 * VW) {
+      const V a = *reinterpret_cast<const V*>(q + i);
+      const V b = *reinterpret_cast<const V*>(w + i);
+      const T* pa = reinterpret_cast<const T*>(&a);
+      const T* pb = reinterpret_cast<const T*>(&b);
+#pragma unroll
+      for (int e = 0; e < VW; ++e) s += pa[e] * pb[e];
+    }
+  } else {
+    for (int i = lane; i < n_rows; i += 64) s += q[i] * w[i];
   }
-  if (threadIdx.x == 0) est[j] = red[0];
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (lane == 0) est[j] = s;
 }
 
 // Total order used by the argsort: larger value first, ties by smaller index, NaN last.
