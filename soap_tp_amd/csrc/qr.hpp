@@ -21,19 +21,9 @@ namespace soapmi {
 
 constexpr int kQrNb = 32;
 
-// One butterfly stage: lanes whose bit MASK is set keep the upper HALF values, the others the
-// lower HALF, and each adds what its partner (lane ^ MASK) holds for the same positions.
-template <typename T, int HALF, int MASK>
-__device__ __forceinline__ void butterfly_stage(T (&vals)[32], int lane) {
-  const bool upper = (lane & MASK) != 0;
-#pragma unroll
-  for (int c = 0; c < HALF; ++c) {
-    const T send = upper ? vals[c] : vals[c + HALF];
-    const T keep = upper ? vals[c + HALF] : vals[c];
-    vals[c] = keep + __shfl_xor(send, MASK, 64);
-  }
-}
-
+// 32 values per lane are summed over the wavefront by a butterfly: at every stage a lane keeps one
+// half of its values (which half is decided by one bit of its lane number), sends the other half to
+// a partner lane and adds what the partner sends for the half it keeps.
 // The two widest stages (partners 32 and 16 lanes apart) on gfx950's lane-swap instructions:
 // v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second
 // (v_permlane16_swap: the odd 16-lane rows of the first with the even rows of the second), which is

@@ -180,14 +180,6 @@ __global__ __launch_bounds__(256) void gather2d_lds_kernel(const float* __restri
   }
 }
 
-template <typename T>
-__global__ void copy2d_kernel(const T* __restrict__ in, int64_t ldi, T* __restrict__ out, int64_t ldo, int rows,
-                              int cols) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= rows) return;
-  for (int j = blockIdx.y; j < cols; j += gridDim.y) out[i + (int64_t)j * ldo] = in[i + (int64_t)j * ldi];
-}
-
 static inline bool aligned16_columns(const void* p, int64_t ld, int64_t rows) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0 && rows % 4 == 0;
 }
