@@ -198,10 +198,11 @@ def soap_step(
         state["variance"] = torch.zeros(rows, columns)
         gram_ema(state["left_preconditioner"], gradient, preconditioner_beta, "left")
         gram_ema(state["right_preconditioner"], gradient, preconditioner_beta, "right")
-        _, state["left_basis"] = eigh_descending(state["left_preconditioner"], basis_implementation)
-        _, state["right_basis"] = eigh_descending(state["right_preconditioner"], basis_implementation)
-        if bases_override and 0 in bases_override:
-            state["left_basis"], state["right_basis"] = (t.clone() for t in bases_override[0])
+        if bases_override and 0 in bases_override:  # the eigensolves would be discarded: skip them
+            state["left_basis"], state["right_basis"] = (t.clone() for t in bases_override[0][:2])
+        else:
+            _, state["left_basis"] = eigh_descending(state["left_preconditioner"], basis_implementation)
+            _, state["right_basis"] = eigh_descending(state["right_preconditioner"], basis_implementation)
         state["step"] = 0
         return torch.zeros_like(gradient)  # soap.py:268-276
 
@@ -218,11 +219,12 @@ def soap_step(
         if bases_override and step in bases_override:
             # keep the transport semantics, but land on the supplied bases
             momentum = rotate(state["momentum"], state["left_basis"], state["right_basis"], "backward")
-            left_order, _, _ = estimated_order(state["left_preconditioner"], state["left_basis"])
-            right_order, _, _ = estimated_order(state["right_preconditioner"], state["right_basis"])
             override = bases_override[step]
             if len(override) == 4:  # caller also supplies the orders that were used
                 left_order, right_order = override[2], override[3]
+            else:
+                left_order, _, _ = estimated_order(state["left_preconditioner"], state["left_basis"])
+                right_order, _, _ = estimated_order(state["right_preconditioner"], state["right_basis"])
             state["left_basis"], state["right_basis"] = override[0].clone(), override[1].clone()
             state["variance"] = permute(state["variance"], left_order, right_order)
             state["momentum"] = rotate(momentum, state["left_basis"], state["right_basis"], "forward")
