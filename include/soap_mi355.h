@@ -110,6 +110,21 @@ int soapmi_rotate_adam_rotate_f32(const float* gradient, int64_t ldg, float* upd
                                   size_t workspace_bytes, void* stream);
 size_t soapmi_rotate_adam_rotate_workspace_bytes(int64_t rows, int64_t cols);
 
+/* soapmi_rotate_adam_rotate_f32 for callers that cannot allocate device memory (code under HIP
+ * graph capture, serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments without the workspace: the two rows x cols temporaries live in a
+ * static device array inside the library (2 x 4194304 floats = 32 MiB per device, held until the
+ * process ends), so the call is limited to rows * cols <= 4194304 (2048 x 2048, 1024 x 4096, ...)
+ * and returns SOAPMI_INVALID_ARGUMENT beyond that.  It calls no allocation routine; the first
+ * call on a device looks up the array's address there.  All calls on one device share the array:
+ * calls that overlap in time on one device (different streams or threads) race; calls ordered on
+ * one stream do not, and nothing needs clearing between them. */
+int soapmi_rotate_adam_rotate_static_f32(const float* gradient, int64_t ldg, float* update, int64_t ldu,
+                                         const float* ql, int64_t ldql, const float* qr, int64_t ldqr,
+                                         float* momentum, int64_t ldm, float* variance, int64_t ldv, int64_t rows,
+                                         int64_t cols, int64_t step, double beta1, double beta2, double eps,
+                                         void* stream);
+
 /* Plain product C = alpha*op(A)*op(B) + beta*C on the same kernel the entry points above use;
  * exported for tests and roofline measurement. */
 int soapmi_gemm_f32(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const float* a,

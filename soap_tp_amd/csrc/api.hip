@@ -100,6 +100,36 @@ static int side_stream(SideStream** out) {
   return kOk;
 }
 
+// Device memory for the entry point that allocates nothing: two rows x cols temporaries of at most
+// kStaticScratchElements floats each (32 MiB in all), part of the code object, so every device
+// the library runs on holds its own copy from module load to process exit.  In host code the
+// array's name is only a handle for hipGetSymbolAddress: the address of this device's copy is
+// looked up once per device and that pointer is what kernels receive.
+constexpr int64_t kStaticScratchElements = 4194304;
+static __device__ __align__(256) float scratch[2 * kStaticScratchElements];
+static float* g_static_scratch[64];
+
+static int static_scratch_address(float** out) {
+  int dev = 0;
+  SOAPMI_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) {
+    set_error("unsupported device index %d", dev);
+    return kRuntimeError;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_static_scratch[dev]) {
+    void* address = nullptr;
+    SOAPMI_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+    if (!address) {
+      set_error("hipGetSymbolAddress returned a null address for the static scratch");
+      return kRuntimeError;
+    }
+    g_static_scratch[dev] = static_cast<float*>(address);
+  }
+  *out = g_static_scratch[dev];
+  return kOk;
+}
+
 static AdamScalars make_adam_scalars(int64_t step, double beta1, double beta2, double eps_in) {
   AdamScalars s;
   s.beta1 = (float)beta1;
@@ -287,32 +317,19 @@ size_t soapmi_rotate_adam_rotate_workspace_bytes(int64_t rows, int64_t cols) {
   return w.total();
 }
 
-int soapmi_rotate_adam_rotate_f32(const float* gradient, int64_t ldg, float* update, int64_t ldu, const float* ql,
-                                  int64_t ldql, const float* qr, int64_t ldqr, float* momentum, int64_t ldm,
-                                  float* variance, int64_t ldv, int64_t rows, int64_t cols, int64_t step,
-                                  double beta1, double beta2, double eps, void* workspace,
-                                  size_t workspace_bytes, void* stream) {
-  int rc = check_adam_args(step, beta1, beta2, eps);
-  if (rc) return rc;
-  SOAPMI_REQUIRE(gradient && update && ql && qr && momentum && variance, "buffer addresses must be nonzero");
-  SOAPMI_REQUIRE(rows > 0 && cols > 0, "matrix dimensions must be positive");
-  SOAPMI_REQUIRE(ldg >= cols && ldu >= cols, "row-major leading dimensions are too small");
-  SOAPMI_REQUIRE(ldql >= rows && ldqr >= cols && ldm >= rows && ldv >= rows, "leading dimensions are too small");
-  const size_t need = soapmi_rotate_adam_rotate_workspace_bytes(rows, cols);
-  void* ws = nullptr;
-  rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
-  if (rc) return rc;
-  Workspace w(ws, need);
-  float* h = w.take<float>((size_t)rows * cols);
-  float* u = w.take<float>((size_t)rows * cols);
-  hipStream_t s = (hipStream_t)stream;
+// The four chained products of soapmi_rotate_adam_rotate_f32 on two caller- or library-provided
+// rows x cols temporaries.
+static int rotate_adam_rotate_chain(const float* gradient, int64_t ldg, float* update, int64_t ldu, const float* ql,
+                                    int64_t ldql, const float* qr, int64_t ldqr, float* momentum, int64_t ldm,
+                                    float* variance, int64_t ldv, int64_t rows, int64_t cols, int64_t step,
+                                    double beta1, double beta2, double eps, float* h, float* u, hipStream_t s) {
   const int m = (int)rows, n = (int)cols;
   const double bc2 = 1.0 - pow(beta2, (double)step);
   AdamScalars sc = make_adam_scalars(step, beta1, beta2, eps / sqrt(bc2));
 
   // 1. H = QL^T G.  The row-major gradient is the column-major matrix S = G^T (cols x rows, ld ldg),
   //    so op(B) = S^T.
-  rc = gemm<float>(s, 1, 1, m, n, m, 1.0f, ql, ldql, gradient, ldg, 0.0f, h, rows);
+  int rc = gemm<float>(s, 1, 1, m, n, m, 1.0f, ql, ldql, gradient, ldg, 0.0f, h, rows);
   if (rc) return rc;
   // 2. U = adam(H QR): the rotated gradient stays in the accumulators.
   {
@@ -332,6 +349,61 @@ int soapmi_rotate_adam_rotate_f32(const float* gradient, int64_t ldg, float* upd
   if (rc) return rc;
   // 4. update (row-major) = H QR^T, i.e. the column-major cols x rows matrix QR H^T.
   return gemm<float>(s, 0, 1, n, m, n, 1.0f, qr, ldqr, h, rows, 0.0f, update, ldu);
+}
+
+static int check_rotate_adam_rotate_args(const float* gradient, int64_t ldg, float* update, int64_t ldu,
+                                         const float* ql, int64_t ldql, const float* qr, int64_t ldqr,
+                                         float* momentum, int64_t ldm, float* variance, int64_t ldv, int64_t rows,
+                                         int64_t cols, int64_t step, double beta1, double beta2, double eps) {
+  int rc = check_adam_args(step, beta1, beta2, eps);
+  if (rc) return rc;
+  SOAPMI_REQUIRE(gradient && update && ql && qr && momentum && variance, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(rows > 0 && cols > 0, "matrix dimensions must be positive");
+  SOAPMI_REQUIRE(ldg >= cols && ldu >= cols, "row-major leading dimensions are too small");
+  SOAPMI_REQUIRE(ldql >= rows && ldqr >= cols && ldm >= rows && ldv >= rows, "leading dimensions are too small");
+  return kOk;
+}
+
+int soapmi_rotate_adam_rotate_f32(const float* gradient, int64_t ldg, float* update, int64_t ldu, const float* ql,
+                                  int64_t ldql, const float* qr, int64_t ldqr, float* momentum, int64_t ldm,
+                                  float* variance, int64_t ldv, int64_t rows, int64_t cols, int64_t step,
+                                  double beta1, double beta2, double eps, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  int rc = check_rotate_adam_rotate_args(gradient, ldg, update, ldu, ql, ldql, qr, ldqr, momentum, ldm, variance,
+                                         ldv, rows, cols, step, beta1, beta2, eps);
+  if (rc) return rc;
+  const size_t need = soapmi_rotate_adam_rotate_workspace_bytes(rows, cols);
+  void* ws = nullptr;
+  rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
+  if (rc) return rc;
+  Workspace w(ws, need);
+  float* h = w.take<float>((size_t)rows * cols);
+  float* u = w.take<float>((size_t)rows * cols);
+  return rotate_adam_rotate_chain(gradient, ldg, update, ldu, ql, ldql, qr, ldqr, momentum, ldm, variance, ldv, rows,
+                                  cols, step, beta1, beta2, eps, h, u, (hipStream_t)stream);
+}
+
+int soapmi_rotate_adam_rotate_static_f32(const float* gradient, int64_t ldg, float* update, int64_t ldu,
+                                         const float* ql, int64_t ldql, const float* qr, int64_t ldqr,
+                                         float* momentum, int64_t ldm, float* variance, int64_t ldv, int64_t rows,
+                                         int64_t cols, int64_t step, double beta1, double beta2, double eps,
+                                         void* stream) {
+  int rc = check_rotate_adam_rotate_args(gradient, ldg, update, ldu, ql, ldql, qr, ldqr, momentum, ldm, variance,
+                                         ldv, rows, cols, step, beta1, beta2, eps);
+  if (rc) return rc;
+  SOAPMI_REQUIRE(rows * cols <= kStaticScratchElements,
+                 "rows * cols = %lld exceeds the %lld elements the static scratch holds; use "
+                 "soapmi_rotate_adam_rotate_f32 with a caller workspace",
+                 (long long)(rows * cols), (long long)kStaticScratchElements);
+  float* base = nullptr;
+  rc = static_scratch_address(&base);
+  if (rc) return rc;
+  // Both temporaries are written in full (beta = 0 products) before anything reads them, so the
+  // previous call's contents need no clearing.
+  float* h = base;
+  float* u = base + kStaticScratchElements;
+  return rotate_adam_rotate_chain(gradient, ldg, update, ldu, ql, ldql, qr, ldqr, momentum, ldm, variance, ldv, rows,
+                                  cols, step, beta1, beta2, eps, h, u, (hipStream_t)stream);
 }
 
 int soapmi_row_major_to_col_major_f32(const float* in, int64_t ldi, float* out, int64_t ldo, int64_t rows,
