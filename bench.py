@@ -3,17 +3,22 @@
 
     python bench.py [--gpus 1] [--steps 50] [--warmup 11] [--shape 4096x11008] [--rank 128]
 
-A "step" is one ``soap_step`` call on a synthetic low-rank-plus-noise gradient that is already
-resident in HBM.  The warm-up contains the initialising call (Gram matrices + both eigensolves) and,
-by default, ten more steps including one basis refresh, so that the timed region is the
-steady-state schedule of the benchmark configuration: K steps with a refresh every 10.  One JSON line
-is printed; ``value`` is K divided by the time of the timed region, taken with HIP events on the
-stream the kernels run on and bracketed by device synchronisations.
+A "step" is one call of the public ``soap_tp_amd.soap_step`` on a synthetic low-rank-plus-noise
+gradient that is already resident in HBM (generated on the CPU by the oracle's generator, so the
+CPU baseline consumes the same bits, and copied over before anything is timed).  The warm-up
+contains the initialising call (Gram matrices + both eigensolves) and, by default, ten more steps
+including one basis refresh, so that the timed region is the steady-state schedule of the
+benchmark configuration: K steps with a refresh every 10.  One JSON line is printed; ``value`` is K
+divided by the time of the timed region: device synchronisation, HIP event, K ``soap_step`` calls,
+HIP event, device synchronisation (the reference times its step the same way,
+scripts/run_soap_tp_timing_gpu.py:139-165).
 
-``roofline`` describes the dominant kernel, the fp32 MFMA product behind the four rotation products
-of a step (algorithmic flops 4 m n (m+n) per step, 2 m n k per launch); its launches are timed live
-with HIP events inside the timed region.  ``cpu_baseline`` times the CPU oracle (torch/MKL on the
-host cores) on a bounded sample of the same workload.
+Stage times come from a second pass over the same schedule that issues the step's library calls
+one by one with event marks between them.  ``roofline`` describes the dominant kernel, the fp32 MFMA
+product behind the four rotation products of a step (algorithmic flops 4 m n (m+n) per step,
+2 m n k per launch), from that pass's events.  After the timed passes one more step is checked
+against the CPU oracle conditionally on the device's bases (``parity_check``).  ``cpu_baseline``
+times the CPU oracle (torch/MKL on the host cores) on a bounded sample of the same workload.
 """
 from __future__ import annotations
 
@@ -39,14 +44,13 @@ HYPER = dict(preconditioner_beta=0.95, beta1=0.95, beta2=0.95, eps=1e-8, basis_r
 MEASURED_TRAFFIC_BYTES = {"4096x11008": 5.33e9}
 
 
-def device_low_rank_plus_noise(rows, columns, rank, seed, device, noise_std=1e-4):
-    generator = torch.Generator(device=device).manual_seed(seed)
-    U, _ = torch.linalg.qr(torch.randn(rows, rank, generator=generator, device=device))
-    V, _ = torch.linalg.qr(torch.randn(columns, rank, generator=generator, device=device))
-    low, high = math.log(1e-4), math.log(1e-1)
-    s = torch.exp(torch.rand(rank, generator=generator, device=device) * (high - low) + low)
-    noise = torch.randn(rows, columns, generator=generator, device=device)
-    return ((U * s) @ V.T + noise_std * noise).contiguous()
+def gradient_pool(rows, columns, rank, count, device, seed0=42):
+    """`count` gradients from the oracle's CPU generator (seed0 + i), copied to the device."""
+    from oracle import soap_oracle as oracle
+
+    pool = [oracle.low_rank_plus_noise(rows, columns, rank, seed=seed0 + i).to(device) for i in range(count)]
+    torch.cuda.synchronize()
+    return pool
 
 
 class StepTimer:
@@ -61,7 +65,11 @@ class StepTimer:
         return event
 
 
-def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True, shard_dim=1):
+def run_schedule(shape, rank, steps, warmup, device, pool_size=6, interval=10, shard_dim=1, detail=True,
+                 parity=False):
+    """Initialising call + warm-up, then `steps` timed calls of the public soap_step (the headline),
+    then, with `detail`, the same number of steps again through the step's individual library calls
+    with event marks between them (stage times), then, with `parity`, one checked step."""
     import soap_tp_amd
     from soap_tp_amd import soap as soap_module
     from soap_tp_amd.ops import (refresh_bases_and_transport_optimizer_state_,
@@ -69,10 +77,10 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True, s
                                  update_right_preconditioner_2d_block_cyclic_)
 
     rows, columns = shape
-    gradients = [device_low_rank_plus_noise(rows, columns, rank, 42 + i, device) for i in range(pool_size)]
-    torch.cuda.synchronize()
+    gradients = gradient_pool(rows, columns, rank, pool_size, device)
     state = {}
-    kwargs = dict(global_shape=shape, shard_dim=shard_dim, block_size=128, process_grid_shape=GRID, **HYPER)
+    hyper = dict(HYPER, basis_refresh_interval=interval)
+    kwargs = dict(global_shape=shape, shard_dim=shard_dim, block_size=128, process_grid_shape=GRID, **hyper)
 
     init_start = time.perf_counter()
     soap_tp_amd.soap_step(gradients[0], state, **kwargs)
@@ -82,26 +90,35 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True, s
         soap_tp_amd.soap_step(gradients[w % pool_size], state, **kwargs)
     torch.cuda.synchronize()
 
-    # The timed region runs the same three library calls per step as soap_step does, with event
-    # marks between them so that stage times are measured on the kernels' own stream.
+    # ---- headline: the public entry point, nothing else inside the timed region
     timer = StepTimer()
-    marks = []
-    interval = HYPER["basis_refresh_interval"]
-    begin = timer.mark()
+    first_step = int(state["step"]) + 1
     wall_start = time.perf_counter()
+    begin = timer.mark()
     for k in range(steps):
-        gradient = gradients[(warmup + k) % pool_size]
-        if detail:
+        soap_tp_amd.soap_step(gradients[(warmup + k) % pool_size], state, **kwargs)
+    end = timer.mark()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - wall_start) * 1e3
+    total_ms = begin.elapsed_time(end)
+    refreshes = sum(1 for step in range(first_step, first_step + steps) if step % interval == 0)
+    result = {"total_ms": total_ms, "wall_ms": wall_ms, "init_ms": init_ms, "refreshes": refreshes}
+
+    # ---- stage times: the same library calls soap_step makes, with event marks between them
+    if detail:
+        marks = []
+        begin = timer.mark()
+        for k in range(steps):
+            gradient = gradients[(warmup + steps + k) % pool_size]
             step = int(state["step"]) + 1
             t0 = timer.mark()
-            update = soap_module._fused_update(gradient, state, rows, columns, step, HYPER["beta1"], HYPER["beta2"],
-                                               HYPER["eps"])
+            soap_module._fused_update(gradient, state, rows, columns, step, hyper["beta1"], hyper["beta2"], hyper["eps"])
             t1 = timer.mark()
             update_left_preconditioner_2d_block_cyclic_(gradient, state["left_preconditioner"],
-                                                        HYPER["preconditioner_beta"], 128, GRID, shard_dim=shard_dim,
+                                                        hyper["preconditioner_beta"], 128, GRID, shard_dim=shard_dim,
                                                         mirror=False)
             update_right_preconditioner_2d_block_cyclic_(gradient, state["right_preconditioner"],
-                                                         HYPER["preconditioner_beta"], 128, GRID,
+                                                         hyper["preconditioner_beta"], 128, GRID,
                                                          shard_dim=shard_dim, mirror=False)
             t2 = timer.mark()
             refreshed = step % interval == 0
@@ -113,24 +130,54 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, detail=True, s
             t3 = timer.mark()
             state["step"] = step
             marks.append((t0, t1, t2, t3, refreshed))
-        else:
-            soap_tp_amd.soap_step(gradient, state, **kwargs)
-    end = timer.mark()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - wall_start) * 1e3
-    total_ms = begin.elapsed_time(end)
-    result = {"total_ms": total_ms, "wall_ms": wall_ms, "init_ms": init_ms}
-    if detail and marks:
+        end = timer.mark()
+        torch.cuda.synchronize()
         rotate = [a.elapsed_time(b) for a, b, _, _, _ in marks]
         gram = [b.elapsed_time(c) for _, b, c, _, _ in marks]
         refresh = [c.elapsed_time(d) for _, _, c, d, r in marks if r]
         result.update(rotate_ms=statistics.mean(rotate), gram_ms=statistics.mean(gram),
-                      refresh_ms=statistics.mean(refresh) if refresh else None, refreshes=len(refresh))
+                      refresh_ms=statistics.mean(refresh) if refresh else None, detail_refreshes=len(refresh),
+                      detail_total_ms=begin.elapsed_time(end))
+
+    if parity:
+        result["parity_check"] = checked_step(gradients[1], state, kwargs, hyper)
     del state
     return result
 
 
-def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True, full_init=False):
+def checked_step(gradient, state, kwargs, hyper):
+    """One more soap_step on the state the timed passes left, compared with the CPU oracle's
+    arithmetic for that step on the same bits, conditionally on the device's bases."""
+    import soap_tp_amd
+    from oracle import soap_oracle as oracle
+
+    step = int(state["step"]) + 1
+    if step % hyper["basis_refresh_interval"] == 0:  # keep the checked step a plain one
+        soap_tp_amd.soap_step(gradient, state, **kwargs)
+        step += 1
+    momentum, variance = state["momentum"].cpu().clone(), state["variance"].cpu().clone()
+    q_left, q_right = state["left_basis"].cpu(), state["right_basis"].cpu()
+    update = soap_tp_amd.soap_step(gradient, state, **kwargs).cpu()
+    gradient = gradient.cpu()
+    start = time.perf_counter()
+    projected = oracle.rotate(gradient, q_left, q_right, "forward")
+    coordinate = oracle.adam_update(projected, momentum, variance, step, hyper["beta1"], hyper["beta2"],
+                                    hyper["eps"] / math.sqrt(1.0 - hyper["beta2"] ** step))
+    expected = oracle.rotate(coordinate, q_left, q_right, "backward")
+    cpu_ms = (time.perf_counter() - start) * 1e3
+
+    def relative(actual, reference):
+        return ((actual.double() - reference.double()).norm() / reference.double().norm()).item()
+
+    errors = {"update": relative(update, expected), "momentum": relative(state["momentum"].cpu(), momentum),
+              "variance": relative(state["variance"].cpu(), variance)}
+    ok = all(math.isfinite(e) and e <= 1e-4 for e in errors.values())
+    return {"step": step, "relative_frobenius_error": errors, "tolerance": 1e-4, "ok": ok,
+            "what": "the step after the timed passes against the CPU oracle, given the device's bases",
+            "cpu_ms": cpu_ms}
+
+
+def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True, full_init=True):
     """The CPU oracle on a bounded sample: `sample_plain_steps` steady-state steps and one refresh."""
     from oracle import soap_oracle as oracle
 
@@ -159,8 +206,8 @@ def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True, full_init
         start = time.perf_counter()
         oracle.refresh(state)
         refresh_ms = (time.perf_counter() - start) * 1e3
-    # one of the two eigensolves of the initialising call (the smaller side, fp64 solve of -P as the
-    # "elpa" variant does); the larger side only on request, it takes most of a minute
+    # the two eigensolves of the initialising call (fp64 solve of -P as the "elpa" variant does); the
+    # larger side (about 20 s at 11008) can be left out with --cpu-small-init
     init_sizes = [min(rows, columns)] + ([max(rows, columns)] if full_init and rows != columns else [])
     init_ms = {}
     for size in init_sizes:
@@ -187,8 +234,8 @@ def run_layer(device, steps=30, rank=64):
 
     shapes = [(4096, 4096)] * 4 + [(4096, 14336)] * 2 + [(14336, 4096)]
     parameters = [torch.nn.Parameter(torch.zeros(shape, device=device)) for shape in shapes]
-    gradients = {shape: [device_low_rank_plus_noise(shape[0], shape[1], rank, 42 + 1000 * i + t, device)
-                         for t in range(2)] for i, shape in enumerate(dict.fromkeys(shapes))}
+    gradients = {shape: gradient_pool(shape[0], shape[1], rank, 2, device, seed0=42 + 1000 * i)
+                 for i, shape in enumerate(dict.fromkeys(shapes))}
     optimizer = SOAP(parameters, lr=3e-3, betas=(HYPER["beta1"], HYPER["beta2"]),
                      shampoo_beta=HYPER["preconditioner_beta"], eps=HYPER["eps"], weight_decay=0.0,
                      precondition_frequency=HYPER["basis_refresh_interval"])
@@ -274,6 +321,31 @@ def calibration_copies(rows, columns, count, device):
     torch.cuda.synchronize()
 
 
+def gpu_eigensolve_ms(sizes, rank, device):
+    """The initialising eigensolve ("elpa" variant: fp64 solve of -P) of a Gram matrix of each size,
+    timed alone with HIP events (second of two calls)."""
+    from oracle import soap_oracle as oracle
+    from soap_tp_amd.ops import allocate_2d_block_cyclic, initialize_basis_2d_block_cyclic_
+
+    result = {}
+    for size in sizes:
+        gradient = oracle.low_rank_plus_noise(size, size, rank, seed=42).to(device)
+        gram = allocate_2d_block_cyclic((size, size), 128, GRID, device=device)
+        gram.copy_(0.05 * gradient @ gradient.T)
+        basis = allocate_2d_block_cyclic((size, size), 128, GRID, device=device)
+        work = allocate_2d_block_cyclic((size, size), 128, GRID, device=device)
+        values = torch.empty(size, dtype=torch.float32, device=device)
+        for _ in range(2):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            initialize_basis_2d_block_cyclic_(gram, basis, work, values, size, 128, GRID, implementation="elpa")
+            end.record()
+            torch.cuda.synchronize()
+        result[str(size)] = begin.elapsed_time(end)
+        del gradient, gram, basis, work
+    return result
+
+
 def parse_shape(text):
     rows, columns = text.lower().split("x")
     return int(rows), int(columns)
@@ -291,11 +363,12 @@ def main():
                              "code paths)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-other-shapes", action="store_true")
-    parser.add_argument("--cpu-full-init", action="store_true",
-                        help="also time the larger side's initialising eigensolve on the CPU oracle (about a minute)")
-    parser.add_argument("--layer", action="store_true",
-                        help="also run the whole-layer configuration (4 x 4096x4096, 2 x 4096x14336, 1 x 14336x4096, "
-                             "rank 64, 30 steps) through the optimizer wrapper and report it under 'layer'")
+    parser.add_argument("--cpu-small-init", action="store_true",
+                        help="time only the smaller side's initialising eigensolve on the CPU oracle (the larger one "
+                             "takes about 20 s at 11008)")
+    parser.add_argument("--no-layer", action="store_true",
+                        help="skip the whole-layer configuration (4 x 4096x4096, 2 x 4096x14336, 1 x 14336x4096, "
+                             "rank 64, 30 steps through the optimizer wrapper), reported under 'layer'")
     parser.add_argument("--calibration-copies", type=int, default=0,
                         help="run this many layout copies of one rows x columns fp32 matrix (transpose_kernel: "
                              "4*rows*columns bytes read and as many written) before the schedule; the known-size "
@@ -314,7 +387,10 @@ def main():
 
     if args.calibration_copies > 0:
         calibration_copies(rows, columns, args.calibration_copies, device)
-    main_run = run_schedule(args.shape, args.rank, args.steps, args.warmup, device, shard_dim=args.shard_dim)
+    main_run = run_schedule(args.shape, args.rank, args.steps, args.warmup, device, shard_dim=args.shard_dim,
+                            parity=True)
+    if not main_run["parity_check"]["ok"]:
+        sys.exit(f"bench.py: the checked step disagrees with the CPU oracle: {main_run['parity_check']}")
     ms_per_step = main_run["total_ms"] / args.steps
     rotation_flops = 4.0 * rows * columns * (rows + columns)
     gram_flops = 1.0 * rows * columns * (rows + columns)
@@ -340,15 +416,20 @@ def main():
                         f"refresh every {HYPER['basis_refresh_interval']} steps, beta1=beta2=shampoo_beta=0.95, "
                         "eps=1e-8, basis_implementation=elpa (fp64 eigensolve)",
             "schedule": f"{args.warmup} warm-up calls (initialisation + {args.warmup - 1} steps), then {args.steps} "
-                        "timed steps",
+                        f"timed calls of soap_step ({main_run['refreshes']} of them refresh the bases)",
+            "gradients": "generated on the CPU by the oracle's generator (seeds 42..47), resident in HBM before timing",
         },
+        "timed_region": "sync, event, K x soap_tp_amd.soap_step, event, sync",
+        "ms_per_step_in_stage_pass": main_run["detail_total_ms"] / args.steps,
+        "parity_check": main_run["parity_check"],
         "stages_ms": {
             "rotate_adam_rotate": main_run["rotate_ms"],
             "gram_pair": main_run["gram_ms"],
             "plain_step": main_run["rotate_ms"] + main_run["gram_ms"],
             "refresh": main_run["refresh_ms"],
             "initialisation_call": main_run["init_ms"],
-            "refreshes_timed": main_run["refreshes"],
+            "refreshes_timed": main_run["detail_refreshes"],
+            "from": "a second pass over the same schedule, library calls issued one by one with event marks",
         },
         "roofline": {
             "bound": "mfma",
@@ -368,22 +449,31 @@ def main():
     }
     if not args.no_other_shapes:
         others = {}
-        for shape, rank in (((1024, 1024), 32), ((4096, 4096), 64), ((8192, 3584), 128)):
+        for shape, rank, steps, interval in (((1024, 1024), 32, 20, 10), ((4096, 4096), 64, 50, 10),
+                                             ((8192, 3584), 128, 100, 5)):
             if shape == args.shape:
                 continue
-            run = run_schedule(shape, rank, 20, 11, device)
+            run = run_schedule(shape, rank, steps, interval + 1, device, interval=interval)
             flops = 5.0 * shape[0] * shape[1] * (shape[0] + shape[1])
             plain = run["rotate_ms"] + run["gram_ms"]
             others[f"{shape[0]}x{shape[1]}"] = {
-                "steps_per_s": 20 / (run["total_ms"] * 1e-3), "plain_step_ms": plain, "refresh_ms": run["refresh_ms"],
-                "initialisation_call_ms": run["init_ms"], "step_mfma_stages_tflops": flops / (plain * 1e-3) / 1e12,
+                "steps": steps, "refresh_every": interval, "steps_per_s": steps / (run["total_ms"] * 1e-3),
+                "plain_step_ms": plain, "refresh_ms": run["refresh_ms"], "initialisation_call_ms": run["init_ms"],
+                "step_mfma_stages_tflops": flops / (plain * 1e-3) / 1e12,
             }
         line["other_shapes"] = others
     line["hbm_stages"] = hbm_stages(rows, columns, device)
-    if args.layer:
+    if not args.no_layer:
         line["layer"] = run_layer(device)
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.shape, args.rank, full_init=args.cpu_full_init)
+        baseline = cpu_baseline(args.shape, args.rank, full_init=not args.cpu_small_init)
+        gpu_ms = gpu_eigensolve_ms([int(size) for size in baseline["init_eigensolve_ms_by_size"]], args.rank, device)
+        baseline["gpu_eigensolve_ms_by_size"] = gpu_ms
+        baseline["eigensolve_speedup_by_size"] = {
+            size: baseline["init_eigensolve_ms_by_size"][size] / gpu_ms[size] for size in gpu_ms}
+        if baseline["refresh_ms"] is not None and main_run["refresh_ms"]:
+            baseline["refresh_speedup"] = baseline["refresh_ms"] / main_run["refresh_ms"]
+        line["cpu_baseline"] = baseline
     else:
         line["cpu_baseline"] = None
     print(json.dumps(line))

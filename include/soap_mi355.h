@@ -58,11 +58,27 @@ const char* soapmi_last_error(void);
  *       factorisation chain side by side, the smaller one on a stream the library owns, forked from
  *       and joined back into the caller's stream with events; with 1 everything is enqueued on the
  *       caller's stream, one chain after the other.  The results are the same bit for bit.
+ *   "persistent_workgroup_budget"  1..256 (default 256): the QR panel kernel and the
+ *       tridiagonalisation's column kernel need all workgroups of a launch resident together (one per
+ *       256 rows).  The library keeps count of the factorisations that may still be running on a
+ *       device and makes a new one wait on the device (stream-wait on an event, no host
+ *       synchronisation) for earlier ones until the sum of their workgroup counts fits this budget.
+ *       A factorisation larger than the budget runs alone.
  *   "message_spin_limit"  0..4194304 (default 4194304): how many times a workgroup of the QR panel
  *       kernel or of the tridiagonalisation's column kernel polls for another workgroup's message
  *       before it gives up.  Giving up never hangs and never passes silently: the kernels leave,
  *       and the factorisation's output is poisoned with NaN (Q's diagonal, the eigenvalues). */
 int soapmi_set_option(const char* name, int64_t value);
+
+/* Failure reporting of the factorisations.  The reference's bindings throw when ELPA or SLATE
+ * report an error (src/soap_tp/csrc/elpa_bindings.cpp:77-91,149-171); here a factorisation's
+ * kernels are only enqueued when its entry point returns, so a failure found on the device (a
+ * persistent kernel that gave up waiting for a message: the output is then NaN-poisoned) is
+ * reported afterwards: returns 1 if a factorisation that has finished on the current device
+ * since the last call with clear != 0 failed, 0 if none did, <0 on error.  Reads a word of pinned
+ * host memory that the device writes: no synchronisation, so it reflects the kernels that have
+ * completed so far. */
+int soapmi_device_error_flag(int clear);
 
 /* ---- Gram preconditioner EMA ---------------------------------------------------------- */
 
@@ -154,7 +170,7 @@ int soapmi_column_dots_f32(const float* q, int64_t ldq, const float* work, int64
                            float* estimates, void* stream);
 
 /* order <- argsort(keys, descending) as int64 (factorizations.py:271).  Ties are broken by the
- * smaller index, NaNs sort last.  Workspace is only used above 16384 keys. */
+ * smaller index, NaNs sort first (torch's descending order).  Workspace is only used above 16384 keys. */
 int soapmi_argsort_desc_f32(const float* keys, int64_t n, int64_t* order, void* workspace, size_t workspace_bytes,
                             void* stream);
 size_t soapmi_argsort_workspace_bytes(int64_t n);

@@ -109,6 +109,15 @@ def call(name: str, *arguments) -> None:
     check(getattr(library(), name)(*arguments))
 
 
+def device_error_flag(clear: bool = True) -> bool:
+    """True if a factorisation that has finished on the current device failed on the device since
+    the flag was last cleared (its output is NaN-poisoned).  Does not synchronise."""
+    code = library().soapmi_device_error_flag(1 if clear else 0)
+    if code < 0:
+        check(code)
+    return code > 0
+
+
 def compiled_gpu_backend() -> str:
     return library().soapmi_compiled_gpu_backend().decode()
 

@@ -20,6 +20,14 @@ def _current_stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+def _workspace(query: str, *sizes):
+    """Scratch for one call from torch's caching allocator: stream-ordered, so the call neither
+    allocates through the runtime nor synchronises, and concurrent streams do not share it."""
+    nbytes = getattr(_native.library(), query)(*sizes)
+    buffer = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=torch.device("cuda", torch.cuda.current_device()))
+    return buffer
+
+
 def _check_grid(process_rows: int, process_cols: int) -> None:
     if process_rows <= 0 or process_cols <= 0 or process_rows * process_cols != 1:
         raise ValueError("process grid must be positive and contain every MPI world rank")
@@ -49,7 +57,8 @@ class NativeBinding:
             raise ValueError("SLATE buffer addresses must be nonzero")
         if n <= 0 or ldmatrix <= 0 or ldq <= 0 or block_size <= 0:
             raise ValueError("matrix size, leading dimensions, and block size must be positive")
-        _native.call("soapmi_qr_f32", matrix, q, n, ldmatrix, ldq, None, 0, _current_stream())
+        work = _workspace("soapmi_qr_workspace_bytes", n)
+        _native.call("soapmi_qr_f32", matrix, q, n, ldmatrix, ldq, work.data_ptr(), work.numel(), _current_stream())
 
     def _rotation(self, forward, q_left, matrix, q_right, rows, columns, ldq_left, ldmatrix, ldq_right,
                   block_size, process_rows, process_cols):
@@ -58,8 +67,9 @@ class NativeBinding:
             raise ValueError("SLATE buffer addresses must be nonzero")
         if min(rows, columns, ldq_left, ldmatrix, ldq_right, block_size) <= 0:
             raise ValueError("matrix dimensions, leading dimensions, and block size must be positive")
+        work = _workspace("soapmi_rotate_workspace_bytes", rows, columns)
         _native.call("soapmi_rotate_f32", q_left, matrix, q_right, rows, columns, ldq_left, ldmatrix,
-                     ldq_right, 1 if forward else 0, None, 0, _current_stream())
+                     ldq_right, 1 if forward else 0, work.data_ptr(), work.numel(), _current_stream())
 
     def slate_forward_rotation_float(self, q_left, matrix, q_right, rows, columns, ldq_left, ldmatrix,
                                      ldq_right, block_size, process_rows, process_cols):
@@ -86,8 +96,9 @@ class NativeBinding:
         if local_rows != n or local_columns != n:
             raise ValueError("on a 1x1 process grid the local shape must equal the matrix size")
         with torch.cuda.device(gpu_id):
-            _native.call("soapmi_eigh_f64", a, eigenvalues, q, n, local_rows, local_rows, None, 0,
-                         _current_stream())
+            work = _workspace("soapmi_eigh_workspace_bytes", n, 8)
+            _native.call("soapmi_eigh_f64", a, eigenvalues, q, n, local_rows, local_rows, work.data_ptr(),
+                         work.numel(), _current_stream())
 
     elpa_eigenvectors_2d_block_cyclic_double = initialize_basis_2d_block_cyclic_
 

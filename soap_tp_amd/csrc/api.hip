@@ -100,6 +100,122 @@ static int side_stream(SideStream** out) {
   return kOk;
 }
 
+// One word of pinned host memory per device that the factorisations' last kernel raises when a
+// persistent kernel gave up waiting for a message (the output is NaN-poisoned then).  The host reads
+// it without synchronising: soapmi_device_error_flag.
+static int* g_report[64];
+
+static int device_report(int** out) {
+  int dev = 0;
+  SOAPMI_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) {
+    set_error("unsupported device index %d", dev);
+    return kRuntimeError;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_report[dev]) {
+    void* p = nullptr;
+    SOAPMI_HIP(hipHostMalloc(&p, 64, hipHostMallocDefault));
+    memset(p, 0, 64);
+    g_report[dev] = static_cast<int*>(p);
+  }
+  *out = g_report[dev];
+  return kOk;
+}
+
+// Persistent kernels (the QR panel kernel, the tridiagonalisation's column kernel) wait inside the
+// kernel for messages from the other workgroups of their launch, so all workgroups of a launch must
+// be resident together.  One launch always is (at most 128 workgroups on 256 compute units), but
+// several factorisations running side by side on different streams could each hold part of the
+// chip while waiting for workgroups that find no free slot.  The library therefore keeps, per
+// device, the workgroup counts of the factorisations that may still be running (an event marks the
+// end of each) and makes a new one wait, on the device, for earlier ones until the sum fits the
+// budget.  Host-side enqueueing of factorisations is serialised per device for the time of the
+// call, which keeps the bookkeeping simple; nothing here synchronises the host with the device.
+static std::atomic<int> g_persistent_budget{256};
+
+struct PersistentLease {
+  hipEvent_t done = nullptr;
+  int workgroups = 0;
+  bool active = false;
+};
+struct PersistentLedger {
+  std::recursive_mutex enqueue;
+  PersistentLease leases[32];
+};
+static PersistentLedger g_ledger[64];
+
+class PersistentGuard {
+ public:
+  PersistentGuard() = default;
+  PersistentGuard(const PersistentGuard&) = delete;
+  PersistentGuard& operator=(const PersistentGuard&) = delete;
+  ~PersistentGuard() {
+    if (ledger_) {
+      if (lease_) lease_->active = false;  // left without release(): nothing was recorded
+      ledger_->enqueue.unlock();
+    }
+  }
+  // Call before the first launch of a factorisation whose persistent kernels have up to `workgroups`
+  // workgroups, on the stream it will run on.
+  int acquire(hipStream_t stream, int workgroups) {
+    int dev = 0;
+    SOAPMI_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) {
+      set_error("unsupported device index %d", dev);
+      return kRuntimeError;
+    }
+    ledger_ = &g_ledger[dev];
+    ledger_->enqueue.lock();
+    stream_ = stream;
+    const int budget = g_persistent_budget.load();
+    int in_flight = 0;
+    PersistentLease* free_slot = nullptr;
+    for (PersistentLease& lease : ledger_->leases) {
+      if (lease.active && hipEventQuery(lease.done) == hipSuccess) lease.active = false;
+      if (lease.active) in_flight += lease.workgroups;
+      else if (!free_slot) free_slot = &lease;
+    }
+    (void)hipGetLastError();  // hipEventQuery reports "not ready" through the error state
+    // Wait (on the device) for earlier factorisations until this one fits; also when no slot is
+    // free.  A factorisation this one waits for never runs beside it, so the two together hold at
+    // most the larger of their counts at any time: the waited-for entry is folded into this one.
+    int held = workgroups;
+    for (PersistentLease& lease : ledger_->leases) {
+      if (in_flight + held <= budget && free_slot) break;
+      if (!lease.active) continue;
+      SOAPMI_HIP(hipStreamWaitEvent(stream, lease.done, 0));
+      in_flight -= lease.workgroups;
+      if (lease.workgroups > held) held = lease.workgroups;
+      lease.active = false;
+      if (!free_slot) free_slot = &lease;
+    }
+    lease_ = free_slot;
+    if (!lease_->done) SOAPMI_HIP(hipEventCreateWithFlags(&lease_->done, hipEventDisableTiming));
+    lease_->workgroups = held;
+    lease_->active = true;
+    return kOk;
+  }
+  // Call after the last launch of the factorisation.
+  int release() {
+    if (!lease_) return kOk;
+    PersistentLease* lease = lease_;
+    lease_ = nullptr;
+    hipError_t e = hipEventRecord(lease->done, stream_);
+    if (e != hipSuccess) {
+      lease->active = false;
+      set_error("hipEventRecord failed: %s", hipGetErrorString(e));
+      return kRuntimeError;
+    }
+    return kOk;
+  }
+
+ private:
+  PersistentLedger* ledger_ = nullptr;
+  PersistentLease* lease_ = nullptr;
+  hipStream_t stream_ = nullptr;
+};
+
 // Device memory for the entry point that allocates nothing: two rows x cols temporaries of at most
 // kStaticScratchElements floats each (32 MiB in all), part of the code object, so every device
 // the library runs on holds its own copy from module load to process exit.  In host code the
@@ -168,8 +284,16 @@ static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_
   Workspace w(ws, need);
   EighWorkspace<T> ews;
   eigh_workspace_layout<T>(w, n, &ews);
-  return eigh_ascending<T>((hipStream_t)stream, a, lda, eigenvalues, q, ldq, (int)n, ews,
-                           g_message_spin_limit.load());
+  int* report = nullptr;
+  rc = device_report(&report);
+  if (rc) return rc;
+  PersistentGuard guard;
+  rc = guard.acquire((hipStream_t)stream, (int)ceil_div64(n, 256));
+  if (rc) return rc;
+  rc = eigh_ascending<T>((hipStream_t)stream, a, lda, eigenvalues, q, ldq, (int)n, ews, g_message_spin_limit.load(),
+                         report);
+  const int rc_release = guard.release();
+  return rc ? rc : rc_release;
 }
 
 extern "C" {
@@ -182,6 +306,16 @@ void soapmi_world_rank_and_size(int* rank, int* size) {
 }
 
 const char* soapmi_last_error(void) { return last_error(); }
+
+int soapmi_device_error_flag(int clear) {
+  int* report = nullptr;
+  int rc = device_report(&report);
+  if (rc) return rc;
+  volatile int* word = report;
+  const int raised = *word != 0 ? 1 : 0;
+  if (clear) *word = 0;
+  return raised;
+}
 
 int soapmi_set_option(const char* name, int64_t value) {
   SOAPMI_REQUIRE(name, "option name must not be null");
@@ -199,6 +333,11 @@ int soapmi_set_option(const char* name, int64_t value) {
   if (strcmp(name, "message_spin_limit") == 0) {
     SOAPMI_REQUIRE(value >= 0 && value <= (int64_t)kQrSpinLimit, "message_spin_limit must be in 0..%u", kQrSpinLimit);
     g_message_spin_limit.store((unsigned)value);
+    return kOk;
+  }
+  if (strcmp(name, "persistent_workgroup_budget") == 0) {
+    SOAPMI_REQUIRE(value >= 1 && value <= 256, "persistent_workgroup_budget must be in 1..256");
+    g_persistent_budget.store((int)value);
     return kOk;
   }
   if (strcmp(name, "refresh_streams") == 0) {
@@ -576,9 +715,17 @@ int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t 
   Workspace w(ws, need);
   QrWorkspace<float> qws;
   qr_workspace_layout<float>(w, n, &qws);
-  return qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws,
-                                     g_qr_persistent_max_wg.load(), g_message_spin_limit.load(),
-                                     g_qr_columns_per_round.load());
+  int* report = nullptr;
+  rc = device_report(&report);
+  if (rc) return rc;
+  PersistentGuard guard;
+  rc = guard.acquire((hipStream_t)stream, (int)ceil_div64(n, 256));
+  if (rc) return rc;
+  rc = qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws,
+                                   g_qr_persistent_max_wg.load(), g_message_spin_limit.load(),
+                                   g_qr_columns_per_round.load(), report);
+  const int rc_release = guard.release();
+  return rc ? rc : rc_release;
 }
 
 size_t soapmi_power_iteration_qr_workspace_bytes(int64_t n) {

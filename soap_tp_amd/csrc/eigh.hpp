@@ -43,12 +43,14 @@ static inline size_t eigh_workspace_bytes(int64_t n) {
 }
 
 // w[0..n) and the diagonal of Z <- NaN if the tridiagonalisation reported lost messages: the
-// decomposition is then unusable, and this makes it impossible to miss.
+// decomposition is then unusable, and this makes it impossible to miss.  The host-visible report
+// word (pinned host memory, may be null) is raised as well.
 template <typename T>
 __global__ void eigh_poison_on_error_kernel(T* __restrict__ w, T* __restrict__ Z, int64_t ldz, int n,
-                                            const int* __restrict__ error) {
+                                            const int* __restrict__ error, int* __restrict__ report) {
   if (*error == 0) return;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (report && i == 0) *report = 1;
   if (i < n) {
     w[i] = T(NAN);
     Z[i + (int64_t)i * ldz] = T(NAN);
@@ -58,7 +60,8 @@ __global__ void eigh_poison_on_error_kernel(T* __restrict__ w, T* __restrict__ Z
 // A (n x n, lower triangle referenced, destroyed) = Z diag(w) Z^T, w ascending.
 template <typename T>
 static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, int64_t ldz, int n,
-                                 const EighWorkspace<T>& ws, unsigned spin_limit = kQrSpinLimit) {
+                                 const EighWorkspace<T>& ws, unsigned spin_limit = kQrSpinLimit,
+                                 int* report = nullptr) {
   if (n <= 0) return kOk;
   int rc = sytrd_lower<T>(s, A, lda, n, ws.d, ws.e, ws.tau, ws.trd, spin_limit);
   if (rc) return rc;
@@ -84,7 +87,7 @@ static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, i
     if (rc) return rc;
   }
   hipLaunchKernelGGL((eigh_poison_on_error_kernel<T>), dim3((unsigned)ceil_div64(n, 256)), dim3(256), 0, s, w, Z, ldz, n,
-                     ws.trd.error);
+                     ws.trd.error, report);
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }

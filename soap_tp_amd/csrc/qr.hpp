@@ -667,11 +667,15 @@ __global__ __launch_bounds__(32 * larft_groups<T>()) void larft32_kernel(const T
   }
 }
 
-// Fills the diagonal of Q with NaN if the error flag is set.
+// Fills the diagonal of Q with NaN if the error flag is set, and raises the host-visible report
+// word (pinned host memory, may be null) so that the host can learn of the failure without
+// reading Q.
 template <typename T>
-__global__ void poison_on_error_kernel(T* __restrict__ Q, int64_t ldq, int n, const int* __restrict__ error) {
+__global__ void poison_on_error_kernel(T* __restrict__ Q, int64_t ldq, int n, const int* __restrict__ error,
+                                       int* __restrict__ report) {
   if (*error == 0) return;
   for (int i = threadIdx.x; i < n; i += blockDim.x) Q[i + (int64_t)i * ldq] = T(NAN);
+  if (report && threadIdx.x == 0) *report = 1;
 }
 
 template <typename T>
@@ -990,7 +994,8 @@ static inline size_t qr_workspace_bytes(int64_t n) {
 template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
                                        const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
-                                       unsigned spin_limit = kQrSpinLimit, int columns_per_round = kQrRoundMax) {
+                                       unsigned spin_limit = kQrSpinLimit, int columns_per_round = kQrRoundMax,
+                                       int* report = nullptr) {
   const int NB = kQrNb, OB = kBrMax;
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
@@ -1098,7 +1103,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
   }
   // A panel kernel that gave up waiting leaves garbage behind: make that impossible to miss.
   hipLaunchKernelGGL((poison_on_error_kernel<T>), dim3(1), dim3(64), 0, s, Qout, ldq, n,
-                     reinterpret_cast<const int*>(ws.sync + 1));
+                     reinterpret_cast<const int*>(ws.sync + 1), report);
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }

@@ -38,25 +38,26 @@ __global__ __launch_bounds__(256) void coldot_kernel(const T* __restrict__ Q, in
   if (lane == 0) est[j] = s;
 }
 
-// Total order used by the argsort: larger value first, ties by smaller index, NaN last.
-// (torch.argsort(descending=True) leaves the order of ties unspecified: factorizations.py:271.)
+// Total order used by the argsort: NaN first (torch.argsort(descending=True) treats NaN as the
+// largest value), then larger value first, ties by smaller index (torch leaves the order of ties
+// unspecified: factorizations.py:271).
 __device__ __forceinline__ bool sorts_before(float va, int ia, float vb, int ib) {
   const bool na = va != va, nb = vb != vb;
-  if (na || nb) return (!na && nb) || (na == nb && ia < ib);
+  if (na || nb) return (na && !nb) || (na == nb && ia < ib);
   if (va > vb) return true;
   if (va < vb) return false;
   return ia < ib;
 }
 
 // Argsort by counting, for up to kArgsortRankMax keys: every workgroup holds all keys in LDS (mapped
-// to unsigned integers that order like sorts_before: larger value first, -0 = +0, NaN last) and each
+// to unsigned integers that order like sorts_before: NaN first, larger value first, -0 = +0) and each
 // key's four threads count the keys that sort before it; that count is the key's position.  n^2 integer
 // comparisons spread over 4n threads, no exchanges and no atomics: about a tenth of the time of a
 // bitonic network run by one workgroup at n = 11008.
 constexpr int kArgsortRankMax = 16384;
 
 __device__ __forceinline__ unsigned argsort_key(float v) {
-  if (v != v) return 0u;
+  if (v != v) return 0xffffffffu;
   unsigned u = __float_as_uint(v);
   if (u == 0x80000000u) u = 0u;  // -0 ties with +0
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
@@ -80,7 +81,8 @@ __global__ __launch_bounds__(256) void argsort_desc_rank_kernel(const float* __r
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int jj = j + e;
-      // padding entries (jj >= n) carry key 0 and an index above every real one: never before a real key
+      // padding entries (jj >= n) carry key 0, below every real key (-inf maps to 0x007fffff), and an
+      // index above every real one: never before a real key
       before += (kk[e] > mine || (kk[e] == mine && jj < i)) ? 1 : 0;
     }
   }
@@ -93,7 +95,7 @@ __global__ __launch_bounds__(256) void argsort_desc_rank_kernel(const float* __r
 __global__ void argsort_init_kernel(const float* __restrict__ keys, int n, int np2, float* v, int* id) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= np2) return;
-  v[i] = (i < n) ? keys[i] : __int_as_float(0x7fc00000);
+  v[i] = (i < n) ? keys[i] : __int_as_float(0xff800000);  // padding: -inf with an index above every real one
   id[i] = i;
 }
 __global__ void argsort_stage_kernel(float* v, int* id, int np2, int k, int j) {

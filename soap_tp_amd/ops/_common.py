@@ -20,6 +20,23 @@ def scratch(nbytes: int, device) -> Tensor:
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
 
+def raise_on_device_error(device) -> None:
+    """Raise if a factorisation enqueued earlier on ``device`` has since failed there.
+
+    The persistent panel kernels of the QR and of the tridiagonalisation bound their waits for
+    other workgroups' messages; a kernel that gives up NaN-poisons its output and raises a word of
+    pinned host memory, which is read here without synchronising.  The reference's bindings throw
+    from inside the call (src/soap_tp/csrc/elpa_bindings.cpp:77-91); here the kernels are still
+    queued when the call returns, so the failure surfaces at the next call on that device."""
+    with torch.cuda.device(device):
+        if _native.device_error_flag(clear=True):
+            raise RuntimeError(
+                "a QR or eigensolver kernel enqueued earlier on this device gave up waiting for a message "
+                "from another workgroup; the bases it produced are NaN-poisoned and the optimizer state "
+                "that used them is invalid. Re-initialise the state (or restore a checkpoint)."
+            )
+
+
 def require_device_tensor(name: str, tensor: Tensor) -> None:
     """The kernels run on the GPU only; same rule and wording as the reference's backend check
     (src/soap_tp/ops/factorizations.py:33-48 with backend 'rocm')."""

@@ -69,11 +69,15 @@ def rotate_2d_block_cyclic_(
                 if direction == "forward"
                 else binding.slate_backward_rotation_float
             )
+            # an injected binding may work on streams of its own (SLATE does): the call is
+            # bracketed by synchronisations, as in the reference (:169,:183)
+            torch.cuda.synchronize(matrix.device)
             function(
                 Q_left.data_ptr(), matrix.data_ptr(), Q_right.data_ptr(), rows, columns,
                 Q_left.stride(1), matrix.stride(1), Q_right.stride(1), block_size,
                 process_rows, process_columns,
             )
+            torch.cuda.synchronize(matrix.device)
     return matrix
 
 
@@ -114,10 +118,12 @@ def estimated_eigenvalue_order_2d_block_cyclic_(
             native_call("soapmi_symm_f32", preconditioner.data_ptr(), Q.data_ptr(), work.data_ptr(), size,
                         preconditioner.stride(1), Q.stride(1), work.stride(1), stream)
         else:
+            torch.cuda.synchronize(device)  # reference :234,:245
             binding.slate_symmetric_multiply_float(
                 preconditioner.data_ptr(), Q.data_ptr(), work.data_ptr(), size,
                 preconditioner.stride(1), block_size, process_rows, process_columns,
             )
+            torch.cuda.synchronize(device)
         native_call("soapmi_column_dots_f32", Q.data_ptr(), Q.stride(1), work.data_ptr(), work.stride(1),
                     size, size, estimates.data_ptr(), stream)
         sort_work = scratch(native_library().soapmi_argsort_workspace_bytes(size), device)
@@ -152,10 +158,12 @@ def qr_2d_block_cyclic_(
             native_call("soapmi_qr_f32", matrix.data_ptr(), Q.data_ptr(), size, matrix.stride(1), Q.stride(1),
                         work.data_ptr(), work.numel(), stream_of(matrix))
         else:
+            torch.cuda.synchronize(matrix.device)  # reference :308,:319
             binding.slate_qr_float(
                 matrix.data_ptr(), Q.data_ptr(), size, matrix.stride(1), Q.stride(1), block_size,
                 process_rows, process_columns,
             )
+            torch.cuda.synchronize(matrix.device)
     return Q
 
 
@@ -257,19 +265,24 @@ def initialize_basis_2d_block_cyclic_(
     binding = validated_binding(elpa_binding, device, rank, world_size)
     with torch.cuda.device(device):
         if elpa_binding is not None and implementation == "elpa":
-            # the reference's staging (:500-546) around the injected solver
-            _symmetrize(preconditioner, size)
-            work.copy_(preconditioner).neg_()
+            # the reference's staging (:500-546) around the injected solver; the preconditioner
+            # itself is left untouched, only its lower triangle is read
+            work.copy_(torch.tril(preconditioner))
+            work.add_(torch.tril(preconditioner, -1).T).neg_()
             work_double = torch.empty_strided(work.size(), work.stride(), dtype=torch.float64, device=device)
             work_double.copy_(work)
             Q_double = torch.empty_strided(Q.size(), Q.stride(), dtype=torch.float64, device=device)
             eigenvalues_double = torch.empty_like(eigenvalues, dtype=torch.float64)
             gpu_id = device.index if device.index is not None else torch.cuda.current_device()
             process_rows, process_columns = process_grid_shape
+            # an injected binding may run on a stream of its own (ELPA does): bracket the call with
+            # synchronisations, as the reference does (:530,:543)
+            torch.cuda.synchronize(device)
             binding.elpa_eigenvectors_2d_block_cyclic_double(
                 work_double.data_ptr(), eigenvalues_double.data_ptr(), Q_double.data_ptr(), size, size, size,
                 block_size, process_rows, process_columns, gpu_id,
             )
+            torch.cuda.synchronize(device)
             Q.copy_(Q_double)
             eigenvalues.copy_(eigenvalues_double).neg_()
             return Q

@@ -37,7 +37,8 @@ from .ops import (
     update_left_preconditioner_2d_block_cyclic_,
     update_right_preconditioner_2d_block_cyclic_,
 )
-from .ops._common import native_call, native_library, require_device_tensor, scratch, stream_of
+from .ops._common import (native_call, native_library, raise_on_device_error, require_device_tensor, scratch,
+                          stream_of)
 from .ops._utils import current_world
 
 STATE_BUFFERS = (
@@ -131,6 +132,7 @@ def soap_step(
     require_device_tensor("gradient_shard", gradient_shard)
     mirror = preconditioner_storage == "full"
     device = gradient_shard.device
+    raise_on_device_error(device)
     initializing = "left_basis" not in state
 
     if initializing:

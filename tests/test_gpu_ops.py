@@ -243,16 +243,110 @@ def test_lost_messages_poison_the_result_instead_of_hanging(device):
         torch.cuda.synchronize()
         return factor.cpu(), values.cpu()
 
+    assert not _native.device_error_flag(clear=True)
     try:
         _native.call("soapmi_set_option", b"message_spin_limit", 0)
         factor, values = run()
     finally:
         _native.call("soapmi_set_option", b"message_spin_limit", 1 << 22)
+        reported = _native.device_error_flag(clear=True)  # cleared: later tests start clean
     assert torch.isnan(factor).any() or relative_l2(factor, expected_q) <= 5e-5
     assert torch.isnan(values).all() or relative_l2(values, expected_values) <= 1e-12
+    # the host learns of a failure without looking at the data: the report word is up exactly when
+    # something was poisoned
+    assert reported == bool(torch.isnan(factor).any() or torch.isnan(values).any())
     factor, values = run()
     assert relative_l2(factor, expected_q) <= 5e-5
     assert relative_l2(values, expected_values) <= 1e-12
+    assert not _native.device_error_flag(clear=True)
+
+
+def test_soap_step_raises_after_a_factorisation_failed_on_the_device(device):
+    """A refresh whose QR gives up (spin limit 0, several workgroups) leaves NaN-poisoned bases; the
+    next call of soap_step on that device must raise instead of computing with them.  If every
+    message happened to be there at the first poll nothing failed and nothing may be raised."""
+    import soap_tp_amd
+    from soap_tp_amd import _native
+    shape = (700, 520)
+    generator = torch.Generator().manual_seed(SEED + 79)
+    state = {}
+    kwargs = dict(global_shape=shape, shard_dim=1, block_size=128, process_grid_shape=GRID, basis_refresh_interval=2)
+    assert not _native.device_error_flag(clear=True)
+    for _ in range(2):
+        soap_tp_amd.soap_step(torch.randn(*shape, generator=generator).to(device), state, **kwargs)
+    try:
+        _native.call("soapmi_set_option", b"message_spin_limit", 0)
+        soap_tp_amd.soap_step(torch.randn(*shape, generator=generator).to(device), state, **kwargs)  # refreshes
+        torch.cuda.synchronize()
+    finally:
+        _native.call("soapmi_set_option", b"message_spin_limit", 1 << 22)
+    poisoned = bool(torch.isnan(state["left_basis"]).any() or torch.isnan(state["right_basis"]).any())
+    gradient = torch.randn(*shape, generator=generator).to(device)
+    if poisoned:
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            soap_tp_amd.soap_step(gradient, state, **kwargs)
+    else:
+        soap_tp_amd.soap_step(gradient, state, **kwargs)
+    assert not _native.device_error_flag(clear=True)  # raising cleared it
+
+
+@pytest.mark.parametrize("budget", [256, 20])
+def test_factorisations_on_several_streams_share_the_chip_safely(budget, device):
+    """Four QR factorisations of 4096 x 4096 matrices (16 workgroups each in their panel kernels) and
+    two eigensolves enqueued back to back on separate streams.  With the default budget of resident
+    persistent workgroups all of them fit side by side; with a budget of 20 each has to wait, on the
+    device, for the one before.  Either way every result must equal the one computed alone, bit for
+    bit, and nothing may be reported as failed."""
+    from soap_tp_amd import _native
+    size = 4096
+    matrices = [make_matrix(size, size, seed=SEED + 300 + i) for i in range(4)]
+    symmetric = [make_preconditioner(2048, SEED + 400 + i).double() for i in range(2)]
+
+    def qr_on(stream, matrix):
+        with torch.cuda.stream(stream):
+            factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+            ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
+        return factor
+
+    def eigh_on(stream, matrix):
+        n = matrix.shape[0]
+        with torch.cuda.stream(stream):
+            a = column_major(matrix, device)
+            values = torch.empty(n, dtype=torch.float64, device=device)
+            vectors = torch.empty(n, n, dtype=torch.float64, device=device).T
+            nbytes = _native.library().soapmi_eigh_workspace_bytes(n, 8)
+            work = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            _native.call("soapmi_eigh_f64", a.data_ptr(), values.data_ptr(), vectors.data_ptr(), n, a.stride(1),
+                         vectors.stride(1), work.data_ptr(), nbytes, stream.cuda_stream)
+        return values, vectors, work, a
+
+    main = torch.cuda.current_stream(device)
+    alone = [qr_on(main, matrix) for matrix in matrices]
+    alone_eigh = [eigh_on(main, matrix)[:2] for matrix in symmetric]
+    torch.cuda.synchronize()
+    assert not _native.device_error_flag(clear=True)
+    streams = [torch.cuda.Stream(device=device) for _ in range(6)]
+    try:
+        _native.call("soapmi_set_option", b"persistent_workgroup_budget", budget)
+        together = [qr_on(stream, matrix) for stream, matrix in zip(streams, matrices)]
+        together_eigh = [eigh_on(stream, matrix) for stream, matrix in zip(streams[4:], symmetric)]
+        torch.cuda.synchronize()
+    finally:
+        _native.call("soapmi_set_option", b"persistent_workgroup_budget", 256)
+    assert not _native.device_error_flag(clear=True)
+    for expected, actual in zip(alone, together):
+        assert torch.isfinite(actual).all()
+        assert torch.equal(expected, actual)
+    for (values, vectors), result in zip(alone_eigh, together_eigh):
+        assert torch.equal(values, result[0]) and torch.equal(vectors, result[1])
+    # and one of them against the oracle
+    q = together[0].double()
+    a = matrices[0].double().to(device)
+    identity_error = q.T @ q
+    identity_error.diagonal().sub_(1.0)
+    assert identity_error.abs().max().item() <= 1e-4
+    r = torch.triu(q.T @ a)
+    assert ((a - q @ r).norm(dim=0) / a.norm(dim=0)).max().item() <= 2e-5
 
 
 def test_argsort_ties_and_large(device):
@@ -268,13 +362,15 @@ def test_argsort_ties_and_large(device):
         _native.call("soapmi_argsort_desc_f32", keys_dev.data_ptr(), count, order.data_ptr(), work.data_ptr(),
                      work.numel(), torch.cuda.current_stream().cuda_stream)
         assert order.tolist() == torch.argsort(keys, descending=True, stable=True).tolist()
-    # signed zeros tie, infinities order like numbers, NaNs go last in index order
+    # NaNs go first in index order (as torch.argsort(descending=True) places them), signed zeros tie,
+    # infinities order like numbers
     special = torch.tensor([0.0, float("nan"), -0.0, float("inf"), -1.0, float("-inf"), 0.0, float("nan"), 2.5, -0.0])
     order = torch.empty(special.numel(), dtype=torch.int64, device=device)
     special_dev = special.to(device)
     _native.call("soapmi_argsort_desc_f32", special_dev.data_ptr(), special.numel(), order.data_ptr(), None, 0,
                  torch.cuda.current_stream().cuda_stream)
-    assert order.tolist() == [3, 8, 0, 2, 6, 9, 4, 5, 1, 7]
+    assert order.tolist() == [1, 7, 3, 8, 0, 2, 6, 9, 4, 5]
+    assert order.tolist() == torch.argsort(special, descending=True, stable=True).tolist()
 
 
 # ---- refresh (tests/unit/test_factorizations.py:501-613) -----------------------------------------

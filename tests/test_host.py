@@ -181,3 +181,42 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     monkeypatch.setattr(_native, "LIBRARY_PATH", tmp_path / "libsoap_mi355.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _native.library()
+
+
+def test_reference_import_paths_resolve_to_this_package():
+    """Every module path the reference's tests and scripts import (tests/unit/*.py,
+    scripts/run_soap_tp_timing_gpu.py:76 of the reference) resolves under the ``soap_tp`` alias to
+    the same objects as in ``soap_tp_amd``."""
+    import importlib
+
+    import soap_tp
+    import soap_tp_amd
+    from soap_tp import elpa_bindings, slate_bindings, soap_step
+    from soap_tp.ops._utils import allocate_2d_block_cyclic, validate_2d_block_cyclic_buffer
+    from soap_tp.ops.factorizations import (initialize_basis_2d_block_cyclic_, power_iteration_qr_2d_block_cyclic_,
+                                            refresh_bases_and_transport_optimizer_state_)
+    from soap_tp.ops.optimizer import adam_update
+    from soap_tp.ops.preconditioners import (update_left_preconditioner_2d_block_cyclic_,
+                                             update_right_preconditioner_2d_block_cyclic_)
+    from soap_tp.soap import soap_step as soap_step_again
+
+    assert soap_step is soap_tp_amd.soap_step is soap_step_again
+    assert soap_tp.ops is soap_tp_amd.ops
+    for path in ("ops", "ops._utils", "ops.factorizations", "ops.optimizer", "ops.preconditioners", "soap"):
+        assert importlib.import_module(f"soap_tp.{path}") is importlib.import_module(f"soap_tp_amd.{path}")
+    assert adam_update is soap_tp_amd.ops.adam_update
+    assert allocate_2d_block_cyclic is soap_tp_amd.ops.allocate_2d_block_cyclic
+    assert initialize_basis_2d_block_cyclic_ is soap_tp_amd.ops.initialize_basis_2d_block_cyclic_
+    assert power_iteration_qr_2d_block_cyclic_ is soap_tp_amd.ops.power_iteration_qr_2d_block_cyclic_
+    assert refresh_bases_and_transport_optimizer_state_ is soap_tp_amd.ops.refresh_bases_and_transport_optimizer_state_
+    assert update_left_preconditioner_2d_block_cyclic_ is soap_tp_amd.ops.update_left_preconditioner_2d_block_cyclic_
+    assert update_right_preconditioner_2d_block_cyclic_ is soap_tp_amd.ops.update_right_preconditioner_2d_block_cyclic_
+    assert callable(validate_2d_block_cyclic_buffer)
+    # the binding modules expose the reference's function names
+    for name in ("compiled_gpu_backend", "mpi_world_rank_and_size", "slate_symmetric_multiply_float", "slate_qr_float",
+                 "slate_forward_rotation_float", "slate_backward_rotation_float"):
+        assert callable(getattr(slate_bindings, name))
+    for name in ("compiled_gpu_backend", "mpi_world_rank_and_size", "initialize_basis_2d_block_cyclic_",
+                 "elpa_eigenvectors_2d_block_cyclic_double"):
+        assert callable(getattr(elpa_bindings, name))
+    assert slate_bindings.compiled_gpu_backend() == "rocm" and elpa_bindings.mpi_world_rank_and_size() == (0, 1)
