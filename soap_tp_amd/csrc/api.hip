@@ -38,6 +38,8 @@ static std::atomic<unsigned> g_message_spin_limit{kQrSpinLimit};
 static std::atomic<int> g_qr_columns_per_round{kQrRoundMax};
 // streams a basis refresh uses: 2 = the two factorisation chains side by side, 1 = one after the other
 static std::atomic<int> g_refresh_streams{2};
+// tridiagonalisation of the eigensolver: kEighOneStage or kEighTwoStage (see soapmi_set_option)
+static std::atomic<int> g_eigh_algorithm{kEighOneStage};
 static std::mutex g_scratch_mutex;
 
 static int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out) {
@@ -277,13 +279,14 @@ static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_
   SOAPMI_REQUIRE(n > 0, "matrix dimensions and block size must be positive");
   SOAPMI_REQUIRE(lda >= n && ldq >= n, "leading dimensions are too small");
   SOAPMI_REQUIRE(n <= 32768, "matrix size %lld exceeds the supported maximum 32768", (long long)n);
-  const size_t need = eigh_workspace_bytes<T>(n);
+  const int algorithm = g_eigh_algorithm.load();
+  const size_t need = eigh_workspace_bytes<T>(n, algorithm);
   void* ws = nullptr;
   int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
   if (rc) return rc;
   Workspace w(ws, need);
   EighWorkspace<T> ews;
-  eigh_workspace_layout<T>(w, n, &ews);
+  eigh_workspace_layout<T>(w, n, &ews, algorithm);
   int* report = nullptr;
   rc = device_report(&report);
   if (rc) return rc;
@@ -291,7 +294,7 @@ static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_
   rc = guard.acquire((hipStream_t)stream, (int)ceil_div64(n, 256));
   if (rc) return rc;
   rc = eigh_ascending<T>((hipStream_t)stream, a, lda, eigenvalues, q, ldq, (int)n, ews, g_message_spin_limit.load(),
-                         report);
+                         report, algorithm);
   const int rc_release = guard.release();
   return rc ? rc : rc_release;
 }
@@ -338,6 +341,11 @@ int soapmi_set_option(const char* name, int64_t value) {
   if (strcmp(name, "persistent_workgroup_budget") == 0) {
     SOAPMI_REQUIRE(value >= 1 && value <= 256, "persistent_workgroup_budget must be in 1..256");
     g_persistent_budget.store((int)value);
+    return kOk;
+  }
+  if (strcmp(name, "eigh_algorithm") == 0) {
+    SOAPMI_REQUIRE(value == kEighOneStage || value == kEighTwoStage, "eigh_algorithm must be 1 (one-stage) or 2 (two-stage)");
+    g_eigh_algorithm.store((int)value);
     return kOk;
   }
   if (strcmp(name, "refresh_streams") == 0) {
@@ -840,7 +848,8 @@ int soapmi_refresh_f32(float* momentum, int64_t ldm, float* variance, int64_t ld
 // ---- eigensolver ------------------------------------------------------------------------------
 
 size_t soapmi_eigh_workspace_bytes(int64_t n, int element_bytes) {
-  return element_bytes == 8 ? eigh_workspace_bytes<double>(n) : eigh_workspace_bytes<float>(n);
+  const int algorithm = g_eigh_algorithm.load();
+  return element_bytes == 8 ? eigh_workspace_bytes<double>(n, algorithm) : eigh_workspace_bytes<float>(n, algorithm);
 }
 
 int soapmi_eigh_f64(double* a, double* eigenvalues, double* q, int64_t n, int64_t lda, int64_t ldq,
@@ -859,12 +868,12 @@ size_t soapmi_initialize_basis_workspace_bytes(int64_t n, int implementation) {
     w.take<double>((size_t)n * n);
     w.take<double>((size_t)n * n);
     w.take<double>((size_t)n);
-    w.take<char>(eigh_workspace_bytes<double>(n));
+    w.take<char>(eigh_workspace_bytes<double>(n, g_eigh_algorithm.load()));
   } else {
     w.take<float>((size_t)n * n);
     w.take<float>((size_t)n * n);
     w.take<float>((size_t)n);
-    w.take<char>(eigh_workspace_bytes<float>(n));
+    w.take<char>(eigh_workspace_bytes<float>(n, g_eigh_algorithm.load()));
   }
   return w.total();
 }
@@ -890,7 +899,7 @@ int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* ei
     double* a64 = w.take<double>((size_t)n * n);
     double* z64 = w.take<double>((size_t)n * n);
     double* w64 = w.take<double>((size_t)n);
-    const size_t eb = eigh_workspace_bytes<double>(n);
+    const size_t eb = eigh_workspace_bytes<double>(n, g_eigh_algorithm.load());
     char* ebuf = w.take<char>(eb);
     // work <- -P (both triangles), then its float64 copy, as factorizations.py:500-507 stages them
     hipLaunchKernelGGL((sym_convert_kernel<float, float>), grid, dim3(256), 0, s, p, ldp, work, ldw, (int)n, -1.0f, 0.0f);
@@ -905,7 +914,7 @@ int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* ei
     float* a32 = w.take<float>((size_t)n * n);
     float* z32 = w.take<float>((size_t)n * n);
     float* w32 = w.take<float>((size_t)n);
-    const size_t eb = eigh_workspace_bytes<float>(n);
+    const size_t eb = eigh_workspace_bytes<float>(n, g_eigh_algorithm.load());
     char* ebuf = w.take<char>(eb);
     hipLaunchKernelGGL((sym_convert_kernel<float, float>), grid, dim3(256), 0, s, p, ldp, a32, n, (int)n, 1.0f, 1e-30f);
     SOAPMI_LAUNCH_CHECK();

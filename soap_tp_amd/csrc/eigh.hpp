@@ -8,8 +8,12 @@
 #include "qr.hpp"
 #include "stedc.hpp"
 #include "sytrd.hpp"
+#include "twostage.hpp"
 
 namespace soapmi {
+
+// Which tridiagonalisation the eigensolver uses.
+enum : int { kEighOneStage = 1, kEighTwoStage = 2 };
 
 template <typename T>
 struct EighWorkspace {
@@ -20,10 +24,11 @@ struct EighWorkspace {
   DcWorkspace<T> dc;
   BlockReflectorWs<T> br;  // block-reflector scratch for the back-transformation
   T* t_block;              // kBrMax x kBrMax
+  TwoStageWorkspace<T> ts; // only laid out for the two-stage algorithm
 };
 
 template <typename T, class WS>
-static inline void eigh_workspace_layout(WS& ws, int64_t n, EighWorkspace<T>* out) {
+static inline void eigh_workspace_layout(WS& ws, int64_t n, EighWorkspace<T>* out, int algorithm = kEighOneStage) {
   EighWorkspace<T> w;
   w.d = ws.template take<T>(n);
   w.e = ws.template take<T>(n);
@@ -32,13 +37,14 @@ static inline void eigh_workspace_layout(WS& ws, int64_t n, EighWorkspace<T>* ou
   dc_workspace_layout<T>(ws, n, out ? &w.dc : nullptr);
   block_reflector_layout<T>(ws, n, out ? &w.br : nullptr);
   w.t_block = ws.template take<T>(kBrMax * kBrMax);
+  if (algorithm == kEighTwoStage) two_stage_workspace_layout<T>(ws, n, out ? &w.ts : nullptr);
   if (out) *out = w;
 }
 
 template <typename T>
-static inline size_t eigh_workspace_bytes(int64_t n) {
+static inline size_t eigh_workspace_bytes(int64_t n, int algorithm = kEighOneStage) {
   WorkspaceSizer sizer;
-  eigh_workspace_layout<T>(sizer, n, nullptr);
+  eigh_workspace_layout<T>(sizer, n, nullptr, algorithm);
   return sizer.total();
 }
 
@@ -57,12 +63,51 @@ __global__ void eigh_poison_on_error_kernel(T* __restrict__ w, T* __restrict__ Z
   }
 }
 
+// out[i, j] = (Tout) in[i, reverse ? n-1-j : j]
+template <typename Tin, typename Tout>
+__global__ void convert_columns_kernel(const Tin* __restrict__ in, int64_t ldi, Tout* __restrict__ out, int64_t ldo,
+                                       int n, int reverse) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  for (int j = blockIdx.y; j < n; j += gridDim.y) {
+    const int sj = reverse ? n - 1 - j : j;
+    out[i + (int64_t)j * ldo] = (Tout)in[i + (int64_t)sj * ldi];
+  }
+}
+
+// The two-stage variant of eigh_ascending: dense -> band -> tridiagonal, divide and conquer, two
+// back-transformations (twostage.hpp).  No persistent kernels: nothing here waits inside a kernel.
+template <typename T>
+static inline int eigh_ascending_two_stage(hipStream_t s, T* A, int64_t lda, T* w, T* Z, int64_t ldz, int n,
+                                           const EighWorkspace<T>& ws) {
+  const TwoStageWorkspace<T>& ts = ws.ts;
+  int rc = sy2sb_lower<T>(s, A, lda, n, ts, ws.br, ws.t_block);
+  if (rc) return rc;
+  hipLaunchKernelGGL((sb_pack_band_kernel<T>), dim3((unsigned)ceil_div64(n, 4)), dim3(256), 0, s, A, lda, n, ts.ab);
+  SOAPMI_LAUNCH_CHECK();
+  rc = sb2st<T>(s, n, ts, ws.d, ws.e);
+  if (rc) return rc;
+  hipLaunchKernelGGL((fill_zero_wide_kernel<T>), dim3(4096), dim3(256), 0, s, ts.zpad, ts.ldz * (int64_t)n);
+  SOAPMI_LAUNCH_CHECK();
+  rc = stedc<T>(s, n, ws.d, ws.e, w, ts.zpad, ts.ldz, ws.dc);
+  if (rc) return rc;
+  rc = sb_apply_q2<T>(s, n, ts);
+  if (rc) return rc;
+  rc = sb_apply_q1<T>(s, A, lda, n, ts, ws.br, ws.t_block);
+  if (rc) return rc;
+  hipLaunchKernelGGL((convert_columns_kernel<T, T>), dim3((unsigned)ceil_div64(n, 256), (unsigned)(n < 4096 ? n : 4096)),
+                     dim3(256), 0, s, ts.zpad, ts.ldz, Z, ldz, n, 0);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
 // A (n x n, lower triangle referenced, destroyed) = Z diag(w) Z^T, w ascending.
 template <typename T>
 static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, int64_t ldz, int n,
                                  const EighWorkspace<T>& ws, unsigned spin_limit = kQrSpinLimit,
-                                 int* report = nullptr) {
+                                 int* report = nullptr, int algorithm = kEighOneStage) {
   if (n <= 0) return kOk;
+  if (algorithm == kEighTwoStage && n >= 3) return eigh_ascending_two_stage<T>(s, A, lda, w, Z, ldz, n, ws);
   int rc = sytrd_lower<T>(s, A, lda, n, ws.d, ws.e, ws.tau, ws.trd, spin_limit);
   if (rc) return rc;
   rc = stedc<T>(s, n, ws.d, ws.e, w, Z, ldz, ws.dc);
@@ -104,18 +149,6 @@ __global__ void sym_convert_kernel(const Tin* __restrict__ in, int64_t ldi, Tout
     Tout v = scale * (Tout)in[r + (int64_t)c * ldi];
     if (i == j) v += diag_shift;
     out[i + (int64_t)j * ldo] = v;
-  }
-}
-
-// out[i, j] = (Tout) in[i, reverse ? n-1-j : j]
-template <typename Tin, typename Tout>
-__global__ void convert_columns_kernel(const Tin* __restrict__ in, int64_t ldi, Tout* __restrict__ out, int64_t ldo,
-                                       int n, int reverse) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  for (int j = blockIdx.y; j < n; j += gridDim.y) {
-    const int sj = reverse ? n - 1 - j : j;
-    out[i + (int64_t)j * ldo] = (Tout)in[i + (int64_t)sj * ldi];
   }
 }
 

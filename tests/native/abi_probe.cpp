@@ -3,6 +3,7 @@
 //   abi_probe [rows cols [repeats [copies]]]
 //   abi_probe qr n          QR of a pseudo-random n x n matrix (library-owned workspace), Q checked on the host
 //   abi_probe eigh n        fp64 eigendecomposition of a symmetric n x n matrix, checked on the host
+//   abi_probe eigh n [timed] two-stage   the eigh modes with the two-stage tridiagonalisation
 //   abi_probe qr|eigh n timed   the same call four times, the last three timed, no host check (the
 //                               check is cubic on one core: minutes at n = 11008)
 //
@@ -163,6 +164,11 @@ static int check_eigh(int64_t n, bool timed_only) {
 }
 
 int main(int argc, char** argv) {
+  // a trailing "two-stage" selects the two-stage tridiagonalisation for the eigh modes
+  if (argc >= 4 && std::string(argv[1]) == "eigh" && std::string(argv[argc - 1]) == "two-stage") {
+    ABI_OK(soapmi_set_option("eigh_algorithm", 2));
+    --argc;
+  }
   const bool timed_only = argc == 4 && std::string(argv[3]) == "timed";
   if ((argc == 3 || timed_only) && std::string(argv[1]) == "qr") return check_qr(std::atoll(argv[2]), timed_only);
   if ((argc == 3 || timed_only) && std::string(argv[1]) == "eigh") return check_eigh(std::atoll(argv[2]), timed_only);

@@ -18,6 +18,16 @@ GRID = (1, 1)
 BLOCK = 2
 
 
+@pytest.fixture(autouse=True, params=[1, 2], ids=["one-stage", "two-stage"])
+def eigh_algorithm(request):
+    """Every test of this module runs with both tridiagonalisations behind the eigensolver entry
+    points: the one-stage reduction (the default) and the two-stage one (dense -> band ->
+    tridiagonal, option "eigh_algorithm" = 2)."""
+    _native.call("soapmi_set_option", b"eigh_algorithm", request.param)
+    yield request.param
+    _native.call("soapmi_set_option", b"eigh_algorithm", 1)
+
+
 def _initialize(preconditioner, implementation, device, poison_upper=False):
     size = preconditioner.shape[0]
     packed = column_major(preconditioner, device)
@@ -71,7 +81,7 @@ def test_initialize_basis_gram_matrices(shape, side, implementation, device):
         torch.testing.assert_close(mine, theirs, rtol=2e-4, atol=2e-4)
 
 
-@pytest.mark.parametrize("size", [1, 2, 3, 5, 31, 32, 33, 64, 100, 257, 1000])
+@pytest.mark.parametrize("size", [1, 2, 3, 5, 31, 32, 33, 34, 64, 66, 100, 257, 600, 1000])
 @pytest.mark.parametrize("implementation", ["elpa", "eigh"])
 def test_initialize_basis_sizes(size, implementation, device):
     g = make_matrix(size, size + 5, seed=SEED + size)
@@ -194,3 +204,32 @@ def test_injected_elpa_binding_follows_reference_staging(device):
     padded = torch.zeros(13, 16, device=device).T[:13]
     with pytest.raises(ValueError, match="exact ELPA leading dimension"):
         ops.initialize_basis_2d_block_cyclic_(packed, basis, padded, values, 13, BLOCK, GRID)
+
+
+def test_two_stage_and_one_stage_agree_at_2048(device):
+    """The two tridiagonalisations on one float64 matrix of size 2048 (64 stage-1 panels, 2046 sweeps of
+    the bulge chase): same spectrum to rounding, both with small residual and orthonormal vectors."""
+    size = 2048
+    gradient = oracle.low_rank_plus_noise(size, size + 512, 32, seed=SEED + 5).double()
+    matrix = 0.05 * gradient @ gradient.T
+    results = []
+    try:
+        for algorithm in (1, 2):
+            _native.call("soapmi_set_option", b"eigh_algorithm", algorithm)
+            a = column_major(torch.tril(matrix), device)
+            q = torch.zeros(size, size, dtype=torch.float64, device=device).T
+            w = torch.zeros(size, dtype=torch.float64, device=device)
+            nbytes = _native.library().soapmi_eigh_workspace_bytes(size, 8)
+            work = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            _native.call("soapmi_eigh_f64", a.data_ptr(), w.data_ptr(), q.data_ptr(), size, size, size, work.data_ptr(),
+                         nbytes, torch.cuda.current_stream().cuda_stream)
+            results.append((w.clone(), q.clone()))
+    finally:
+        _native.call("soapmi_set_option", b"eigh_algorithm", 1)
+    scale = results[0][0].abs().max().item()
+    assert (results[0][0] - results[1][0]).abs().max().item() <= 1e-12 * scale
+    device_matrix = matrix.to(device)
+    for w, q in results:
+        assert torch.all(w[1:] >= w[:-1])
+        assert ((device_matrix @ q - q * w).norm() / device_matrix.norm()).item() <= 1e-13
+        assert (q.T @ q - torch.eye(size, dtype=torch.float64, device=device)).abs().max().item() <= 1e-12
