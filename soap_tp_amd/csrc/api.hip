@@ -561,7 +561,8 @@ int soapmi_row_major_to_col_major_f32(const float* in, int64_t ldi, float* out, 
   SOAPMI_REQUIRE(ldi >= cols && ldo >= rows, "leading dimensions are too small");
   // `in` is the column-major cols x rows matrix S; out = S^T.
   hipLaunchKernelGGL((transpose_kernel<float>), dim3((unsigned)ceil_div64(cols, 64), (unsigned)ceil_div64(rows, 64)),
-                     dim3(256), 0, (hipStream_t)stream, in, ldi, out, ldo, (int)cols, (int)rows);
+                     dim3(256), 0, (hipStream_t)stream, in, ldi, out, ldo, (int)cols, (int)rows,
+                     transpose_vec_ok<float>(in, ldi, out, ldo, cols, rows));
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
@@ -573,7 +574,8 @@ int soapmi_col_major_to_row_major_f32(const float* in, int64_t ldi, float* out, 
   SOAPMI_REQUIRE(in && out, "buffer addresses must be nonzero");
   SOAPMI_REQUIRE(ldi >= rows && ldo >= cols, "leading dimensions are too small");
   hipLaunchKernelGGL((transpose_kernel<float>), dim3((unsigned)ceil_div64(rows, 64), (unsigned)ceil_div64(cols, 64)),
-                     dim3(256), 0, (hipStream_t)stream, in, ldi, out, ldo, (int)rows, (int)cols);
+                     dim3(256), 0, (hipStream_t)stream, in, ldi, out, ldo, (int)rows, (int)cols,
+                     transpose_vec_ok<float>(in, ldi, out, ldo, rows, cols));
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
@@ -894,6 +896,7 @@ int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* ei
   Workspace w(ws, need);
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)ceil_div64(n, 256), (unsigned)(n < 4096 ? n : 4096));
+  const dim3 tiles((unsigned)ceil_div64(n, 64), (unsigned)ceil_div64(n, 64));
   const unsigned vblocks = (unsigned)ceil_div64(n, 256);
   if (implementation == 0) {
     double* a64 = w.take<double>((size_t)n * n);
@@ -902,8 +905,8 @@ int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* ei
     const size_t eb = eigh_workspace_bytes<double>(n, g_eigh_algorithm.load());
     char* ebuf = w.take<char>(eb);
     // work <- -P (both triangles), then its float64 copy, as factorizations.py:500-507 stages them
-    hipLaunchKernelGGL((sym_convert_kernel<float, float>), grid, dim3(256), 0, s, p, ldp, work, ldw, (int)n, -1.0f, 0.0f);
-    hipLaunchKernelGGL((sym_convert_kernel<float, double>), grid, dim3(256), 0, s, p, ldp, a64, n, (int)n, -1.0, 0.0);
+    hipLaunchKernelGGL((sym_convert_kernel<float, float>), tiles, dim3(256), 0, s, p, ldp, work, ldw, (int)n, -1.0f, 0.0f);
+    hipLaunchKernelGGL((sym_convert_kernel<float, double>), tiles, dim3(256), 0, s, p, ldp, a64, n, (int)n, -1.0, 0.0);
     SOAPMI_LAUNCH_CHECK();
     rc = soapmi_eigh_f64(a64, w64, z64, n, n, n, ebuf, eb, stream);
     if (rc) return rc;
@@ -916,7 +919,7 @@ int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* ei
     float* w32 = w.take<float>((size_t)n);
     const size_t eb = eigh_workspace_bytes<float>(n, g_eigh_algorithm.load());
     char* ebuf = w.take<char>(eb);
-    hipLaunchKernelGGL((sym_convert_kernel<float, float>), grid, dim3(256), 0, s, p, ldp, a32, n, (int)n, 1.0f, 1e-30f);
+    hipLaunchKernelGGL((sym_convert_kernel<float, float>), tiles, dim3(256), 0, s, p, ldp, a32, n, (int)n, 1.0f, 1e-30f);
     SOAPMI_LAUNCH_CHECK();
     rc = soapmi_eigh_f32(a32, w32, z32, n, n, n, ebuf, eb, stream);
     if (rc) return rc;

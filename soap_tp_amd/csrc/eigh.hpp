@@ -138,17 +138,33 @@ static inline int eigh_ascending(hipStream_t s, T* A, int64_t lda, T* w, T* Z, i
 }
 
 // out[i, j] = scale * (T_out) in[max(i,j), min(i,j)] (+ shift on the diagonal): builds the full
-// symmetric solver input from the lower triangle of P, converting precision on the way.
+// symmetric solver input from the lower triangle of P, converting precision on the way.  One
+// workgroup per 64 x 64 tile on or below the diagonal (grid: tiles x tiles, the others return at
+// once): the tile is read with lanes along rows, written as it is and, transposed through LDS,
+// onto its mirror image, so that every access to either matrix is coalesced.
 template <typename Tin, typename Tout>
-__global__ void sym_convert_kernel(const Tin* __restrict__ in, int64_t ldi, Tout* __restrict__ out, int64_t ldo, int n,
-                                   Tout scale, Tout diag_shift) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  for (int j = blockIdx.y; j < n; j += gridDim.y) {
-    const int r = i > j ? i : j, c = i > j ? j : i;
-    Tout v = scale * (Tout)in[r + (int64_t)c * ldi];
-    if (i == j) v += diag_shift;
-    out[i + (int64_t)j * ldo] = v;
+__global__ __launch_bounds__(256) void sym_convert_kernel(const Tin* __restrict__ in, int64_t ldi, Tout* __restrict__ out,
+                                                          int64_t ldo, int n, Tout scale, Tout diag_shift) {
+  __shared__ Tout tile[64][65];
+  const int bi = blockIdx.x, bj = blockIdx.y;
+  if (bi < bj) return;
+  const int r0 = bi * 64, c0 = bj * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int c = ty; c < 64; c += 4) {
+    const int gr = r0 + tx, gc = c0 + c;
+    if (gr < n && gc < n) {
+      const int r = gr > gc ? gr : gc, q = gr > gc ? gc : gr;  // only diagonal tiles hold entries above the diagonal
+      Tout v = scale * (Tout)in[r + (int64_t)q * ldi];
+      if (gr == gc) v += diag_shift;
+      tile[c][tx] = v;
+      out[gr + (int64_t)gc * ldo] = v;
+    }
+  }
+  if (bi == bj) return;
+  __syncthreads();
+  for (int r = ty; r < 64; r += 4) {
+    const int gr = r0 + r, gc = c0 + tx;
+    if (gr < n && gc < n) out[gc + (int64_t)gr * ldo] = tile[tx][r];
   }
 }
 

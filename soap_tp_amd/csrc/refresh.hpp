@@ -122,9 +122,10 @@ __global__ void argsort_finish_kernel(const int* id, int n, int64_t* order) {
 // identity.  Three kernels, chosen by launch_gather2d:
 //   gather2d_columns_kernel  rows not permuted, everything 16-byte aligned: a thread moves four
 //                            consecutive rows of a column per load, eight columns per thread
-//   gather2d_lds_kernel      rows permuted, a source column fits in LDS: a workgroup reads two source
-//                            columns with coalesced loads, then serves its output rows from LDS, so
-//                            the matrix crosses HBM once each way however scattered the row order is
+//   gather2d_lds_kernel      rows permuted, a source column fits in LDS (up to 16384 rows): a workgroup
+//                            reads two source columns (one above 8192 rows) with coalesced loads, then
+//                            serves its output rows from LDS, so the matrix crosses HBM once each way
+//                            however scattered the row order is
 //   gather2d_kernel          anything else (lanes along i: coalesced when rows are not permuted)
 template <typename T>
 __global__ void gather2d_kernel(const T* __restrict__ in, int64_t ldi, T* __restrict__ out, int64_t ldo, int rows,
@@ -159,26 +160,59 @@ __global__ __launch_bounds__(256) void gather2d_columns_kernel(const float* __re
     if (j0 + c < cols) *reinterpret_cast<float4*>(out + i4 + (int64_t)(j0 + c) * ldo) = v[c];
 }
 
-constexpr int kGatherLdsRows = 8192;  // two source columns of this many floats: 64 KB of LDS
+// LDS holds COLS source columns of up to kGatherLdsFloats / COLS rows each (64 KB in all): two
+// columns per workgroup up to 8192 rows, one column up to 16384 rows.  With VEC every global access
+// moves 16 bytes: the source columns are read as float4, and a thread produces four consecutive
+// output rows per store (their four source rows come out of LDS one by one).
+constexpr int kGatherLdsFloats = 16384;
 
+template <int COLS, bool VEC>
 __global__ __launch_bounds__(256) void gather2d_lds_kernel(const float* __restrict__ in, int64_t ldi,
                                                            float* __restrict__ out, int64_t ldo, int rows, int cols,
                                                            const int64_t* __restrict__ row_order,
                                                            const int64_t* __restrict__ col_order) {
-  __shared__ float column[2][kGatherLdsRows];
-  const int j0 = 2 * blockIdx.x;
-  const bool second = j0 + 1 < cols;
-  const int64_t s0 = col_order ? col_order[j0] : (int64_t)j0;
-  const int64_t s1 = second ? (col_order ? col_order[j0 + 1] : (int64_t)(j0 + 1)) : s0;
-  for (int i = threadIdx.x; i < rows; i += 256) {
-    column[0][i] = in[i + s0 * ldi];
-    column[1][i] = in[i + s1 * ldi];
+  constexpr int CAP = kGatherLdsFloats / COLS;
+  __shared__ __attribute__((aligned(16))) float column[COLS][CAP];
+  const int j0 = COLS * blockIdx.x;
+  int64_t src[COLS];
+#pragma unroll
+  for (int c = 0; c < COLS; ++c) {
+    const int j = min(j0 + c, cols - 1);
+    src[c] = col_order ? col_order[j] : (int64_t)j;
+  }
+  if (VEC) {
+    for (int i4 = threadIdx.x * 4; i4 < rows; i4 += 1024) {
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+        *reinterpret_cast<float4*>(&column[c][i4]) = *reinterpret_cast<const float4*>(in + i4 + src[c] * ldi);
+    }
+  } else {
+    for (int i = threadIdx.x; i < rows; i += 256) {
+#pragma unroll
+      for (int c = 0; c < COLS; ++c) column[c][i] = in[i + src[c] * ldi];
+    }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < rows; i += 256) {
-    const int si = (int)row_order[i];
-    out[i + (int64_t)j0 * ldo] = column[0][si];
-    if (second) out[i + (int64_t)(j0 + 1) * ldo] = column[1][si];
+  if (VEC) {
+    for (int i4 = threadIdx.x * 4; i4 < rows; i4 += 1024) {
+      const longlong2 a = *reinterpret_cast<const longlong2*>(row_order + i4);
+      const longlong2 b = *reinterpret_cast<const longlong2*>(row_order + i4 + 2);
+      const int s0 = (int)a.x, s1 = (int)a.y, s2 = (int)b.x, s3 = (int)b.y;
+#pragma unroll
+      for (int c = 0; c < COLS; ++c) {
+        if (j0 + c < cols) {
+          const float4 v = make_float4(column[c][s0], column[c][s1], column[c][s2], column[c][s3]);
+          *reinterpret_cast<float4*>(out + i4 + (int64_t)(j0 + c) * ldo) = v;
+        }
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < rows; i += 256) {
+      const int si = (int)row_order[i];
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+        if (j0 + c < cols) out[i + (int64_t)(j0 + c) * ldo] = column[c][si];
+    }
   }
 }
 
@@ -193,9 +227,22 @@ static inline void launch_gather2d(hipStream_t s, const float* in, int64_t ldi, 
   if (!row_order && aligned16_columns(in, ldi, rows) && aligned16_columns(out, ldo, rows)) {
     const dim3 grid((unsigned)ceil_div64(rows, 1024), (unsigned)ceil_div64(cols, kGatherColsPerThread));
     hipLaunchKernelGGL(gather2d_columns_kernel, grid, dim3(256), 0, s, in, ldi, out, ldo, (int)rows, (int)cols, col_order);
-  } else if (row_order && rows <= kGatherLdsRows) {
-    hipLaunchKernelGGL(gather2d_lds_kernel, dim3((unsigned)ceil_div64(cols, 2)), dim3(256), 0, s, in, ldi, out, ldo,
-                       (int)rows, (int)cols, row_order, col_order);
+  } else if (row_order && rows <= kGatherLdsFloats) {
+    // (row_order comes from an int64 allocation: 16-byte aligned whenever the data pointers are)
+    const bool vec = aligned16_columns(in, ldi, rows) && aligned16_columns(out, ldo, rows) &&
+                     reinterpret_cast<uintptr_t>(row_order) % 16 == 0;
+    const dim3 two((unsigned)ceil_div64(cols, 2)), one((unsigned)cols);
+    if (rows <= kGatherLdsFloats / 2) {
+      if (vec) hipLaunchKernelGGL((gather2d_lds_kernel<2, true>), two, dim3(256), 0, s, in, ldi, out, ldo, (int)rows,
+                                  (int)cols, row_order, col_order);
+      else hipLaunchKernelGGL((gather2d_lds_kernel<2, false>), two, dim3(256), 0, s, in, ldi, out, ldo, (int)rows,
+                              (int)cols, row_order, col_order);
+    } else {
+      if (vec) hipLaunchKernelGGL((gather2d_lds_kernel<1, true>), one, dim3(256), 0, s, in, ldi, out, ldo, (int)rows,
+                                  (int)cols, row_order, col_order);
+      else hipLaunchKernelGGL((gather2d_lds_kernel<1, false>), one, dim3(256), 0, s, in, ldi, out, ldo, (int)rows,
+                              (int)cols, row_order, col_order);
+    }
   } else {
     const dim3 grid((unsigned)ceil_div64(rows, 256), (unsigned)(cols < 8192 ? cols : 8192));
     hipLaunchKernelGGL((gather2d_kernel<float>), grid, dim3(256), 0, s, in, ldi, out, ldo, (int)rows, (int)cols,

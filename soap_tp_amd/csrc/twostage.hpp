@@ -96,6 +96,14 @@ __global__ void sb_extract_tridiagonal_kernel(const T* __restrict__ AB, int n, T
   if (j + 1 < n) e[j] = AB[1 + (int64_t)kSbLd * j];
 }
 
+// Y (rows x nbw, ld ldy) <- the transpose of yt (nbw x rows, ld 32), with its first `lead` rows zero.
+template <typename T>
+__global__ void sb_form_y_kernel(const T* __restrict__ yt, T* __restrict__ Y, int64_t ldy, int nbw, int rows, int lead) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  for (int c = 0; c < nbw; ++c) Y[r + (int64_t)c * ldy] = (r < lead) ? T(0) : yt[c + 32 * (int64_t)r];
+}
+
 // A (n x n, lower triangle referenced) -> band form in place: on exit the band holds Q1^T A Q1
 // (lower part), the stage-1 reflectors lie below it (column j: unit entry at row j + b, vector
 // below), their scalars in ws.tau1.  The upper triangle of A is used as scratch.
@@ -126,48 +134,54 @@ static inline int sy2sb_lower(hipStream_t s, T* A, int64_t lda, int n, const Two
     }
     SOAPMI_LAUNCH_CHECK();
     if (rows <= 1) break;  // nothing below: no trailing matrix to update
+    // The products below start `lead` rows above the first row the reflectors touch, at a multiple
+    // of 128, with V carrying zeros in those rows: for n a multiple of 128 every extent is then a
+    // multiple of the MFMA tile and the products take the fast path.
+    const int lead = (p + b) % 128;
+    const int rows_al = rows + lead;
+    const int r_al = p + b - lead;
     // [V | Y | V]: V in the first and the third slot now, Y below
     T* V = ws.p3;
     T* Y = ws.p3 + (int64_t)nbw * ldp;
     T* V2 = ws.p3 + (int64_t)2 * nbw * ldp;
-    launch_extract_v<T>(s, Ap, lda, rows, p, p, nbw, V, ldp);
-    launch_extract_v<T>(s, Ap, lda, rows, p, p, nbw, V2, ldp);
+    launch_extract_v<T>(s, Ap, lda, rows_al, p - lead, p, nbw, V, ldp, lead);
+    launch_extract_v<T>(s, Ap, lda, rows_al, p - lead, p, nbw, V2, ldp, lead);
     SOAPMI_LAUNCH_CHECK();
     BlockReflectorWs<T> inner = br;
     inner.v = V;
-    int rc = build_t_factor<T>(s, inner, rows, nbw, ldp, ws.tau1 + p, t_block);
+    int rc = build_t_factor<T>(s, inner, rows_al, nbw, ldp, ws.tau1 + p, t_block);
     if (rc) return rc;
     if (nbw < b) {
       // Last block column with fewer rows below the band than columns: the columns [pe, p + b) have no
       // reflector of their own but lie in the rows Q^T acts on: C <- (I - V T^T V^T) C.
-      rc = apply_block_reflector<T>(s, inner, t_block, true, rows, nbw, p + b - pe, ldp, A + (p + b) + (int64_t)pe * lda,
-                                    lda);
+      rc = apply_block_reflector<T>(s, inner, t_block, true, rows_al, nbw, p + b - pe, ldp,
+                                    A + r_al + (int64_t)pe * lda, lda);
       if (rc) return rc;
     }
-    T* A22 = A + (p + b) + (int64_t)(p + b) * lda;
-    // wt = V^T A22 (nbw x rows)
-    rc = gemm<T, Skinny>(s, 1, 0, nbw, rows, rows, T(1), V, ldp, A22, lda, T(0), ws.wt, 32,
-                         split_count(ceil_div64(rows, Skinny::BN), rows, nbw, rows, ldp), br.splitk);
+    T* A22 = A + r_al + (int64_t)r_al * lda;  // the trailing matrix, extended by `lead` rows and columns
+    // wt = V^T A22 (nbw x rows_al); its first `lead` columns belong to no trailing column and are dropped below
+    rc = gemm<T, Skinny>(s, 1, 0, nbw, rows_al, rows_al, T(1), V, ldp, A22, lda, T(0), ws.wt, 32,
+                         split_count(ceil_div64(rows_al, Skinny::BN), rows_al, nbw, rows_al, ldp), br.splitk);
     if (rc) return rc;
     // xt = T^T wt = X^T
-    rc = gemm<T>(s, 1, 0, nbw, rows, nbw, T(1), t_block, kBrMax, ws.wt, 32, T(0), ws.xt, 32);
+    rc = gemm<T>(s, 1, 0, nbw, rows_al, nbw, T(1), t_block, kBrMax, ws.wt, 32, T(0), ws.xt, 32);
     if (rc) return rc;
     // small0 = X^T V = (V^T X)^T ; small1 = small0 T
     T* s0 = ws.small;
     T* s1 = ws.small + 32 * 32;
-    rc = gemm<T, Skinny>(s, 0, 0, nbw, nbw, rows, T(1), ws.xt, 32, V, ldp, T(0), s0, 32,
-                         split_count(1, rows, nbw, nbw, ldp), br.splitk);
+    rc = gemm<T, Skinny>(s, 0, 0, nbw, nbw, rows_al, T(1), ws.xt, 32, V, ldp, T(0), s0, 32,
+                         split_count(1, rows_al, nbw, nbw, ldp), br.splitk);
     if (rc) return rc;
     rc = gemm<T>(s, 0, 0, nbw, nbw, nbw, T(1), s0, 32, t_block, kBrMax, T(0), s1, 32);
     if (rc) return rc;
     // xt <- Y^T = X^T - 1/2 (S^T T) V^T
-    rc = gemm<T>(s, 0, 1, nbw, rows, nbw, T(-0.5), s1, 32, V, ldp, T(1), ws.xt, 32);
+    rc = gemm<T>(s, 0, 1, nbw, rows_al, nbw, T(-0.5), s1, 32, V, ldp, T(1), ws.xt, 32);
     if (rc) return rc;
-    hipLaunchKernelGGL((transpose_kernel<T>), dim3((unsigned)ceil_div64(nbw, 64), (unsigned)ceil_div64(rows, 64)),
-                       dim3(256), 0, s, ws.xt, (int64_t)32, Y, ldp, nbw, rows);
+    hipLaunchKernelGGL((sb_form_y_kernel<T>), dim3((unsigned)ceil_div64(rows_al, 256)), dim3(256), 0, s, ws.xt, Y, ldp,
+                       nbw, rows_al, lead);
     SOAPMI_LAUNCH_CHECK();
     // A22 -= [V | Y] [Y | V]^T
-    rc = gemm<T>(s, 0, 1, rows, rows, 2 * nbw, T(-1), V, ldp, Y, ldp, T(1), A22, lda);
+    rc = gemm<T>(s, 0, 1, rows_al, rows_al, 2 * nbw, T(-1), V, ldp, Y, ldp, T(1), A22, lda);
     if (rc) return rc;
   }
   return kOk;
@@ -494,7 +508,7 @@ static inline int sb_apply_q2(hipStream_t s, int n, const TwoStageWorkspace<T>& 
   const int64_t ldt = n;
   hipLaunchKernelGGL((fill_zero_wide_kernel<T>), dim3(256), dim3(256), 0, s, ws.zt + (int64_t)n * ldt, (int64_t)64 * ldt);
   hipLaunchKernelGGL((transpose_kernel<T>), dim3((unsigned)ceil_div64(n, 64), (unsigned)ceil_div64(n, 64)), dim3(256), 0, s,
-                     ws.zpad, ws.ldz, ws.zt, ldt, n, n);
+                     ws.zpad, ws.ldz, ws.zt, ldt, n, n, transpose_vec_ok<T>(ws.zpad, ws.ldz, ws.zt, ldt, n, n));
   SOAPMI_LAUNCH_CHECK();
   const int t_last = 2 * (groups - 1) + k0;
   for (int t = 0; t <= t_last; ++t) {
@@ -510,7 +524,7 @@ static inline int sb_apply_q2(hipStream_t s, int n, const TwoStageWorkspace<T>& 
   }
   SOAPMI_LAUNCH_CHECK();
   hipLaunchKernelGGL((transpose_kernel<T>), dim3((unsigned)ceil_div64(n, 64), (unsigned)ceil_div64(n, 64)), dim3(256), 0, s,
-                     ws.zt, ldt, ws.zpad, ws.ldz, n, n);
+                     ws.zt, ldt, ws.zpad, ws.ldz, n, n, transpose_vec_ok<T>(ws.zt, ldt, ws.zpad, ws.ldz, n, n));
   SOAPMI_LAUNCH_CHECK();
   return kOk;
 }
