@@ -492,6 +492,127 @@ __global__ __launch_bounds__(256) void sb_apply_blocks_kernel(const T* __restric
   for (int r = 0; r < 63; ++r) zp[(int64_t)r * ldt] = z[r];
 }
 
+// The same time step on the fp64 matrix cores.  A wavefront owns 64 columns of the block's 64-row
+// window (the 63 rows the block touches and one more, whose row of V is zero) and keeps them in the
+// "b" operand layout of v_mfma_f64_16x16x4: register (ks, ct) of lane l holds row 4 ks + l / 16 of
+// column 16 ct + l % 16.  That is also the accumulator layout of the 16-row tile ks / 4, register
+// ks % 4, so the three products chain without a layout change:
+//   W  = V^T Z   "a" = pieces of V^T from LDS, "b" = the window registers
+//   W2 = T W     "a" = pieces of T,            "b" = W's accumulator registers (register r = k step r)
+//   Z -= V W2    "a" = pieces of -V,           "b" = W2's registers, accumulated onto the window registers
+// Tiles of V that lie outside the parallelogram are skipped: columns 16 j .. 16 j + 15 of V have
+// their entries in rows 16 j .. 16 j + 46 only.
+__global__ __launch_bounds__(256) void sb_apply_blocks_mfma_kernel(const double* __restrict__ blk, int n, int t,
+                                                                  int ri_lo, int groups, double* __restrict__ Zt,
+                                                                  int64_t ldt) {
+  constexpr int b = kSbNb, g = kSbNb;
+  using MF = Mfma<double>;
+  __shared__ double Vd[64 * 32];  // Vd[r * 32 + a] = V[r][a]
+  __shared__ double Vn[32 * 64];  // Vn[a * 64 + r] = -V[r][a]
+  __shared__ double Tt[32 * 32];  // Tt[c * 32 + a] = T[a][c]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ri = ri_lo + (int)blockIdx.x;
+  const int gi = groups - 1 - ri, k = t - 2 * ri;
+  const int k0 = (n - 2) / b;
+  const double* src = blk + sb_block_index(gi, k, k0) * kSbBlockStride;
+  for (int e = tid; e < 64 * 32; e += 256) {
+    Vd[e] = 0.0;
+    Vn[e] = 0.0;
+  }
+  __syncthreads();
+  for (int e = tid; e < 32 * 32; e += 256) {
+    const int l = e & 31, a = e >> 5;  // compact form: src[l + 32 a] = V[a + l][a]
+    const double v = src[e];
+    Vd[(a + l) * 32 + a] = v;
+    Vn[a * 64 + a + l] = -v;
+    Tt[e] = src[32 * 32 + e];  // stored as T[a][c] at a + 32 c already
+  }
+  __syncthreads();
+  const int c0 = (blockIdx.y * 4 + wave) * 64;  // this wavefront's first column
+  if (c0 >= n) return;
+  const int64_t r0 = (int64_t)gi * g + 1 + (int64_t)k * b;
+  const int kq = lane >> 4, idx = lane & 15;
+  double* zp = Zt + c0 + idx + (r0 + kq) * ldt;  // + 16 ct + 4 ks ldt
+  // columns beyond n: clamp the address (loads) and skip the store
+  bool live[4];
+#pragma unroll
+  for (int ct = 0; ct < 4; ++ct) live[ct] = c0 + 16 * ct + idx < n;
+  MF::Acc z[4][4];  // z[rt][ct][q]: row 16 rt + 4 q + kq, column 16 ct + idx
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        z[rt][ct][q] = live[ct] ? zp[16 * ct + (int64_t)(16 * rt + 4 * q) * ldt] : 0.0;
+  // W[i][ct] = sum over the rows of V's column tile i: k steps 4 i .. 4 i + 11
+  MF::Acc w[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w[i][ct][q] = 0.0;
+#pragma unroll
+    for (int ks = 4 * i; ks < 4 * i + 12; ++ks) {
+      const double a = Vd[(4 * ks + kq) * 32 + 16 * i + idx];  // V^T[a = 16 i + idx][r = 4 ks + kq]
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) w[i][ct] = MF::mma(a, z[ks >> 2][ct][ks & 3], w[i][ct]);
+    }
+  }
+  // W2 = T W, T upper triangular: tile row 0 needs W's tiles 0 and 1, tile row 1 only tile 1
+  MF::Acc w2[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w2[i][ct][q] = 0.0;
+#pragma unroll
+    for (int j = i; j < 2; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const double a = Tt[(16 * j + 4 * q + kq) * 32 + 16 * i + idx];  // T[16 i + idx][16 j + 4 q + kq]
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) w2[i][ct] = MF::mma(a, w[j][ct][q], w2[i][ct]);
+      }
+    }
+  }
+  // Z -= V W2: row tile rt of V has entries in column tiles j with rt - 2 <= j <= rt
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (j > rt || j < rt - 2) continue;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const double a = Vn[(16 * j + 4 * q + kq) * 64 + 16 * rt + idx];  // -V[16 rt + idx][16 j + 4 q + kq]
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) z[rt][ct] = MF::mma(a, w2[j][ct][q], z[rt][ct]);
+      }
+    }
+  }
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (live[ct]) zp[16 * ct + (int64_t)(16 * rt + 4 * q) * ldt] = z[rt][ct][q];
+}
+
+template <typename T>
+static inline void launch_apply_blocks(hipStream_t s, const T* blk, int n, int t, int ri_lo, int groups, int count, T* Zt,
+                                       int64_t ldt) {
+  if constexpr (std::is_same<T, double>::value) {
+    hipLaunchKernelGGL(sb_apply_blocks_mfma_kernel, dim3(count, (unsigned)ceil_div64(n, 256)), dim3(256), 0, s, blk, n, t,
+                       ri_lo, groups, Zt, ldt);
+  } else {
+    hipLaunchKernelGGL((sb_apply_blocks_kernel<T>), dim3(count, (unsigned)ceil_div64(n, 256)), dim3(256), 0, s, blk, n, t,
+                       ri_lo, groups, Zt, ldt);
+  }
+}
+
 // Z (rows 0 .. n-1 of the padded matrix ws.zpad, ld ws.ldz, n columns) <- Q2 Z.  Works on the
 // transpose (ws.zt) and writes the result back into ws.zpad.
 template <typename T>
@@ -519,8 +640,7 @@ static inline int sb_apply_q2(hipStream_t s, int n, const TwoStageWorkspace<T>& 
     const int ri_lo = std::max(0, bound <= 0 ? 0 : (bound + 2) / 3);
     const int count = ri_hi - ri_lo + 1;
     if (count <= 0) continue;
-    hipLaunchKernelGGL((sb_apply_blocks_kernel<T>), dim3(count, (unsigned)ceil_div64(n, 256)), dim3(256), 0, s, ws.blk, n, t,
-                       ri_lo, groups, ws.zt, ldt);
+    launch_apply_blocks<T>(s, ws.blk, n, t, ri_lo, groups, count, ws.zt, ldt);
   }
   SOAPMI_LAUNCH_CHECK();
   hipLaunchKernelGGL((transpose_kernel<T>), dim3((unsigned)ceil_div64(n, 64), (unsigned)ceil_div64(n, 64)), dim3(256), 0, s,
