@@ -341,3 +341,28 @@ def test_bases_and_refresh_at_14336(shape, device):
     gram = ops.allocate_2d_block_cyclic(state[f"{side}_preconditioner"].shape, BLOCK, GRID, device=device)
     gram.copy_(_full(state[f"{side}_preconditioner"]))
     check_power_iteration_and_qr(gram, state[f"{side}_basis"], 64, device)
+
+
+def test_two_stage_eigensolver_at_4096(device):
+    """The two-stage tridiagonalisation (option "eigh_algorithm" = 2) on the 4096 x 4096 Gram matrix of
+    the benchmark's second configuration, through the basis initialisation: the same invariants as the
+    default solver has to meet, and the same eigenvalues."""
+    from soap_tp_amd import _native
+
+    size, rank = 4096, 64
+    gradient = oracle.low_rank_plus_noise(size, size, rank, seed=SEED).to(device)
+    gram = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+    gram.copy_(0.05 * gradient @ gradient.T)
+    spectra = []
+    try:
+        for algorithm in (1, 2):
+            _native.call("soapmi_set_option", b"eigh_algorithm", algorithm)
+            basis = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+            work = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+            values = torch.empty(size, dtype=torch.float32, device=device)
+            ops.initialize_basis_2d_block_cyclic_(gram, basis, work, values, size, BLOCK, GRID, implementation="elpa")
+            check_eigenbasis(gram, basis, rank, cpu_eigenvalues=(algorithm == 2))
+            spectra.append(values.clone())
+    finally:
+        _native.call("soapmi_set_option", b"eigh_algorithm", 1)
+    assert (spectra[0] - spectra[1]).abs().max().item() <= 1e-6 * spectra[0].abs().max().item()
