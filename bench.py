@@ -72,9 +72,7 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, interval=10, s
     with event marks between them (stage times), then, with `parity`, one checked step."""
     import soap_tp_amd
     from soap_tp_amd import soap as soap_module
-    from soap_tp_amd.ops import (refresh_bases_and_transport_optimizer_state_,
-                                 update_left_preconditioner_2d_block_cyclic_,
-                                 update_right_preconditioner_2d_block_cyclic_)
+    from soap_tp_amd.ops import refresh_bases_and_transport_optimizer_state_
 
     rows, columns = shape
     gradients = gradient_pool(rows, columns, rank, pool_size, device)
@@ -114,12 +112,7 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, interval=10, s
             t0 = timer.mark()
             soap_module._fused_update(gradient, state, rows, columns, step, hyper["beta1"], hyper["beta2"], hyper["eps"])
             t1 = timer.mark()
-            update_left_preconditioner_2d_block_cyclic_(gradient, state["left_preconditioner"],
-                                                        hyper["preconditioner_beta"], 128, GRID, shard_dim=shard_dim,
-                                                        mirror=False)
-            update_right_preconditioner_2d_block_cyclic_(gradient, state["right_preconditioner"],
-                                                         hyper["preconditioner_beta"], 128, GRID,
-                                                         shard_dim=shard_dim, mirror=False)
+            soap_module._fused_gram_pair(gradient, state, rows, columns, hyper["preconditioner_beta"], False)
             t2 = timer.mark()
             refreshed = step % interval == 0
             if refreshed:

@@ -92,6 +92,13 @@ int soapmi_device_error_flag(int clear);
 int soapmi_gram_ema_f32(const float* g, int64_t rows, int64_t cols, int64_t ldg, int g_row_major, int side,
                         float* p, int64_t ldp, float beta, int mirror, void* stream);
 
+/* Both Gram updates of one step (src/soap_tp/soap.py:425-448: the left and the right update with the
+ * same gradient) as one launch: left (rows x rows) <- lerp(left, G G^T, 1-beta) and right
+ * (cols x cols) <- lerp(right, G^T G, 1-beta).  Same arithmetic per element as two calls of
+ * soapmi_gram_ema_f32; the joint grid fills the compute units better than either product alone. */
+int soapmi_gram_ema_pair_f32(const float* g, int64_t rows, int64_t cols, int64_t ldg, int g_row_major, float* left,
+                             int64_t ldl, float* right, int64_t ldr, float beta, int mirror, void* stream);
+
 /* Copies the strictly lower triangle of the n x n matrix P onto its upper triangle. */
 int soapmi_symmetrize_lower_f32(float* p, int64_t n, int64_t ldp, void* stream);
 

@@ -403,6 +403,44 @@ int soapmi_gram_ema_f32(const float* g, int64_t rows, int64_t cols, int64_t ldg,
   return launch_gemm<float>((hipStream_t)stream, prob, epi, 1);
 }
 
+int soapmi_gram_ema_pair_f32(const float* g, int64_t rows, int64_t cols, int64_t ldg, int g_row_major, float* left,
+                             int64_t ldl, float* right, int64_t ldr, float beta, int mirror, void* stream) {
+  SOAPMI_REQUIRE(g && left && right, "buffer addresses must be nonzero");
+  SOAPMI_REQUIRE(rows > 0 && cols > 0, "matrix dimensions must be positive");
+  SOAPMI_REQUIRE(beta >= 0.0f && beta <= 1.0f, "beta must be in [0, 1], got %g.", (double)beta);
+  SOAPMI_REQUIRE(ldg >= (g_row_major ? cols : rows) && ldg > 0, "gradient leading dimension is too small");
+  SOAPMI_REQUIRE(ldl >= rows && ldr >= cols, "preconditioner leading dimension is too small");
+  SOAPMI_REQUIRE(left != right, "the two preconditioners must not overlap");
+  // see soapmi_gram_ema_f32 for the operand transposes of each side
+  const int lta = g_row_major ? 1 : 0, ltb = g_row_major ? 0 : 1;
+  const int rta = ltb, rtb = lta;
+  EpiEmaLower<float> el{left, ldl, 1.0f - beta, mirror}, er{right, ldr, 1.0f - beta, mirror};
+  using Wide = DefaultTile<float>::type;
+  using Small = SmallTile<float>::type;
+  const int64_t tl = ceil_div64(rows, Wide::BM), tr = ceil_div64(cols, Wide::BM);
+  const int64_t tiles = tl * (tl + 1) / 2 + tr * (tr + 1) / 2;  // default tiles of both lower triangles together
+  // the 64 x 64 tile when the default one would fill the compute units badly: few tiles, or a last
+  // round of workgroups that is mostly empty (4096^2: 1056 tiles, a fifth round with 32 of 256)
+  bool small = tiles <= 128;
+  if (!small && tiles < 2048) small = (double)tiles < 0.85 * (double)(ceil_div64(tiles, 256) * 256);
+  int rc = kOk;
+  bool launched;
+  if (small) {
+    GemmProblem<float> pl = make_problem<float, Small>(lta, ltb, (int)rows, (int)rows, (int)cols, g, ldg, g, ldg, true);
+    GemmProblem<float> pr = make_problem<float, Small>(rta, rtb, (int)cols, (int)cols, (int)rows, g, ldg, g, ldg, true);
+    launched = launch_gemm_pair<float, EpiEmaLower<float>, Small>((hipStream_t)stream, pl, el, pr, er, &rc);
+  } else {
+    GemmProblem<float> pl = make_problem<float, Wide>(lta, ltb, (int)rows, (int)rows, (int)cols, g, ldg, g, ldg, true);
+    GemmProblem<float> pr = make_problem<float, Wide>(rta, rtb, (int)cols, (int)cols, (int)rows, g, ldg, g, ldg, true);
+    launched = launch_gemm_pair<float, EpiEmaLower<float>, Wide>((hipStream_t)stream, pl, el, pr, er, &rc);
+  }
+  if (launched) return rc;
+  // a layout pair that has no joint kernel: one launch per side
+  rc = soapmi_gram_ema_f32(g, rows, cols, ldg, g_row_major, 0, left, ldl, beta, mirror, stream);
+  if (rc) return rc;
+  return soapmi_gram_ema_f32(g, rows, cols, ldg, g_row_major, 1, right, ldr, beta, mirror, stream);
+}
+
 int soapmi_symmetrize_lower_f32(float* p, int64_t n, int64_t ldp, void* stream) {
   SOAPMI_REQUIRE(p, "buffer addresses must be nonzero");
   SOAPMI_REQUIRE(n >= 0 && ldp >= n && ldp > 0, "invalid matrix size or leading dimension");

@@ -381,6 +381,16 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi
   gemm_tile_body<T, Cfg, Epi, MODE>(p, epi, blockIdx.x, blockIdx.y);
 }
 
+// Two independent products in one launch: workgroups [0, grid0) take the first problem, the rest
+// the second (each with its own operand-layout mode).  Used for the two Gram updates of a step,
+// whose tile counts together fill the 256 compute units better than either does alone.
+template <typename T, class Cfg, class Epi, int MODE0, int MODE1>
+__global__ __launch_bounds__(Cfg::NT) void gemm_pair_kernel(GemmProblem<T> p0, Epi e0, GemmProblem<T> p1, Epi e1,
+                                                            int grid0) {
+  if ((int)blockIdx.x < grid0) gemm_tile_body<T, Cfg, Epi, MODE0>(p0, e0, blockIdx.x, 0);
+  else gemm_tile_body<T, Cfg, Epi, MODE1>(p1, e1, (int)blockIdx.x - grid0, 0);
+}
+
 // One problem per blockIdx.z, described in device memory (sizes may be produced by earlier
 // kernels of the same stream); workgroups beyond a problem's tile count return at once.
 template <typename T>
@@ -529,6 +539,40 @@ static inline int launch_gemm(hipStream_t stream, const GemmProblem<T>& p, const
   }
   SOAPMI_LAUNCH_CHECK();
   return kOk;
+}
+
+// Fast-path mode of a problem for tile Cfg (see launch_gemm), or -1.
+template <typename T, class Cfg>
+static inline int fast_mode(const GemmProblem<T>& p) {
+  const bool fast = p.vecA && p.vecB && p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0 && p.K > 0 && p.K % Cfg::BK == 0 &&
+                    p.k_chunk % Cfg::BK == 0;
+  return fast ? ((p.transA ? 0 : 1) | (p.transB ? 2 : 0)) : -1;
+}
+
+// Launches two problems (same tile, same epilogue type) as one grid when their mode pair is one of
+// those compiled: (0, 3), (3, 0) -- the two Gram products of one gradient -- or both general.
+// Returns false without launching anything otherwise.
+template <typename T, class Epi, class Cfg>
+static inline bool launch_gemm_pair(hipStream_t stream, const GemmProblem<T>& p0, const Epi& e0,
+                                    const GemmProblem<T>& p1, const Epi& e1, int* rc) {
+  *rc = kOk;
+  if (p0.M <= 0 || p0.N <= 0 || p1.M <= 0 || p1.N <= 0) return false;
+  const int m0 = fast_mode<T, Cfg>(p0), m1 = fast_mode<T, Cfg>(p1);
+  const int grid0 = 8 * ((p0.num_tiles + 7) / 8), grid1 = 8 * ((p1.num_tiles + 7) / 8);
+  const dim3 grid(grid0 + grid1);
+  if (m0 == 0 && m1 == 3)
+    hipLaunchKernelGGL((gemm_pair_kernel<T, Cfg, Epi, 0, 3>), grid, dim3(Cfg::NT), 0, stream, p0, e0, p1, e1, grid0);
+  else if (m0 == 3 && m1 == 0)
+    hipLaunchKernelGGL((gemm_pair_kernel<T, Cfg, Epi, 3, 0>), grid, dim3(Cfg::NT), 0, stream, p0, e0, p1, e1, grid0);
+  else if (m0 == -1 && m1 == -1)
+    hipLaunchKernelGGL((gemm_pair_kernel<T, Cfg, Epi, -1, -1>), grid, dim3(Cfg::NT), 0, stream, p0, e0, p1, e1, grid0);
+  else
+    return false;
+  if (hipGetLastError() != hipSuccess) {
+    set_error("kernel launch failed");
+    *rc = kRuntimeError;
+  }
+  return true;
 }
 
 // C = alpha*op(A)*op(B) + beta*C.  If `partials` is non-null and k_splits > 1 the K range is

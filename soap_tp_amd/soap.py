@@ -81,6 +81,20 @@ def _fused_update(gradient: Tensor, state, rows: int, columns: int, step: int, b
     return update
 
 
+def _fused_gram_pair(gradient: Tensor, state, rows: int, columns: int, beta: float, mirror: bool) -> None:
+    """Both Gram EMAs of a step in one launch (the gradient is the contiguous fp32 copy made by soap_step)."""
+    if not 0.0 <= beta <= 1.0:
+        raise ValueError(f"beta must be in [0, 1], got {beta}.")
+    left, right = state["left_preconditioner"], state["right_preconditioner"]
+    with torch.cuda.device(gradient.device):
+        native_call(
+            "soapmi_gram_ema_pair_f32",
+            gradient.data_ptr(), rows, columns, gradient.stride(0), 1,
+            left.data_ptr(), left.stride(1), right.data_ptr(), right.stride(1),
+            float(beta), 1 if mirror else 0, stream_of(gradient),
+        )
+
+
 @torch.no_grad()
 def soap_step(
     gradient_shard: Tensor,
@@ -145,6 +159,9 @@ def soap_step(
     _profile.dump("gradient", profile_step, gradient)
 
     def update_preconditioners(suffix: str) -> None:
+        if slate_binding is None and not profiling and not initializing:
+            _fused_gram_pair(gradient, state, rows, columns, preconditioner_beta, mirror)
+            return
         update_left_preconditioner_2d_block_cyclic_(
             gradient, state["left_preconditioner"], preconditioner_beta, block_size, process_grid_shape,
             shard_dim=shard_dim, mirror=mirror)

@@ -108,6 +108,35 @@ def test_permute_and_redistribute_are_exact(shape, device):
         ops.permute_2d_block_cyclic_(packed, shape, row_order, column_order[:-1], BLOCK, GRID)
 
 
+@pytest.mark.parametrize("shape", [(8, 12), (13, 9), (96, 160), (256, 384), (1024, 1024), (700, 1300), (2048, 512)])
+@pytest.mark.parametrize("row_major", [True, False])
+@pytest.mark.parametrize("mirror", [True, False])
+def test_gram_pair_equals_the_two_single_updates(shape, row_major, mirror, device):
+    """soapmi_gram_ema_pair_f32 (both Gram updates of a step in one launch) against two calls of
+    soapmi_gram_ema_f32: the same products element by element, so the results are equal bit for bit
+    whichever tile either path picks."""
+    from soap_tp_amd import _native
+    rows, columns = shape
+    gradient = make_matrix(rows, columns, seed=SEED + rows + columns)
+    stored = gradient.to(device) if row_major else column_major(gradient, device)
+    ldg = stored.stride(0) if row_major else stored.stride(1)
+    stream = torch.cuda.current_stream().cuda_stream
+    start_left = column_major(make_preconditioner(rows, SEED + 11), device)
+    start_right = column_major(make_preconditioner(columns, SEED + 12), device)
+    single = [start_left.clone(), start_right.clone()]
+    for side in (0, 1):
+        _native.call("soapmi_gram_ema_f32", stored.data_ptr(), rows, columns, ldg, 1 if row_major else 0, side,
+                     single[side].data_ptr(), single[side].stride(1), 0.9, 1 if mirror else 0, stream)
+    paired = [start_left.clone(), start_right.clone()]
+    _native.call("soapmi_gram_ema_pair_f32", stored.data_ptr(), rows, columns, ldg, 1 if row_major else 0,
+                 paired[0].data_ptr(), paired[0].stride(1), paired[1].data_ptr(), paired[1].stride(1), 0.9,
+                 1 if mirror else 0, stream)
+    for expected, actual in zip(single, paired):
+        assert torch.equal(expected, actual)
+    expected_left = oracle.gram_ema(make_preconditioner(rows, SEED + 11), gradient, 0.9, "left")
+    assert relative_l2(torch.tril(paired[0]), torch.tril(expected_left)) <= RTOL
+
+
 # ---- rotations (tests/unit/test_factorizations.py:376-399) ---------------------------------------
 @pytest.mark.parametrize("shape", MATRIX_SHAPES + ((130, 70), (256, 384)))
 @pytest.mark.parametrize("direction", ["forward", "backward"])
