@@ -14,7 +14,9 @@
 //   back 2   Z <- Q2 Z: the stage-2 reflectors of 32 consecutive sweeps at one position form a
 //            63 x 32 parallelogram that is applied as one compact-WY block; blocks of sweep group i at
 //            position k commute with all blocks that share their "time" 2 (groups - 1 - i) + k, so
-//            every time step is three strided-batch products.
+//            every time step is one launch over (blocks of the step) x (column chunks), on the
+//            transposed eigenvector matrix; in fp64 the three products of a block run on the matrix
+//            cores with the window held in registers.
 //   back 1   Z <- Q1 Z with the stage-1 reflectors, 256 columns per compact-WY block.
 #pragma once
 #include "common.hpp"
