@@ -49,11 +49,12 @@ const char* soapmi_last_error(void);
  *   "qr_persistent_max_workgroups"  0..128 (default 128): a QR panel whose grid (rows / 256) fits
  *       runs as one persistent launch whose workgroups exchange partial sums through device memory;
  *       larger panels, or all panels with 0, run one launch per column instead.
- *   "qr_columns_per_round"  1..4 (default 4): panel columns the persistent QR panel kernel factors per
- *       exchange of partial sums.  The exchange carries the dot products of all the round's columns;
- *       the reflectors after the first follow from those by rank-one corrections (guarded: a
- *       column whose corrected norm shows cancellation ends the round and starts the next one with
- *       directly computed sums); 1 computes every column's sums directly.
+ *   "qr_columns_per_round"  1..4 or 32 (default 32): panel columns the persistent QR panel kernel
+ *       factors per exchange of partial sums.  The exchange carries the dot products of all the
+ *       round's columns; the reflectors after the first follow from those by rank-one corrections
+ *       (guarded: a column whose corrected norm shows cancellation ends the round and starts the
+ *       next one with directly computed sums); 1 computes every column's sums directly; 32 covers
+ *       a whole panel with one exchange of its 32 x 32 Gram matrix, computed on the matrix cores.
  *   "refresh_streams"  1 or 2 (default 2): with 2, soapmi_refresh_f32 runs the left and the right
  *       factorisation chain side by side, the smaller one on a stream the library owns, forked from
  *       and joined back into the caller's stream with events; with 1 everything is enqueued on the

@@ -35,7 +35,7 @@ static std::atomic<int> g_qr_persistent_max_wg{kQrPersistentMaxWg};
 // polls a workgroup spends waiting for another one's message before it gives up (see soapmi_set_option)
 static std::atomic<unsigned> g_message_spin_limit{kQrSpinLimit};
 // panel columns the QR factors per message round (see soapmi_set_option)
-static std::atomic<int> g_qr_columns_per_round{kQrRoundMax};
+static std::atomic<int> g_qr_columns_per_round{kQrWholePanel};
 // streams a basis refresh uses: 2 = the two factorisation chains side by side, 1 = one after the other
 static std::atomic<int> g_refresh_streams{2};
 // tridiagonalisation of the eigensolver: kEighOneStage or kEighTwoStage (see soapmi_set_option)
@@ -329,7 +329,8 @@ int soapmi_set_option(const char* name, int64_t value) {
     return kOk;
   }
   if (strcmp(name, "qr_columns_per_round") == 0) {
-    SOAPMI_REQUIRE(value >= 1 && value <= kQrRoundMax, "qr_columns_per_round must be in 1..%d", kQrRoundMax);
+    SOAPMI_REQUIRE((value >= 1 && value <= kQrRoundMax) || value == kQrWholePanel,
+                   "qr_columns_per_round must be in 1..%d or %d (the whole panel)", kQrRoundMax, kQrWholePanel);
     g_qr_columns_per_round.store((int)value);
     return kOk;
   }

@@ -263,6 +263,43 @@ __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&s
   }
 }
 
+// Waits for and sums, in order, the words base[0], base[stride], ... of the first `count` of COUNT
+// slots and likewise `count3` of EXTRA slots from base3 (every slot is loaded whether it counts or
+// not, so all must be valid memory: the addresses are then constant offsets from two bases, which
+// keeps this many loads in flight within the register budget).  False after too many polls or once
+// the error flag is up.
+template <int COUNT, int STRIDE, int EXTRA, int STRIDE3>
+__device__ __forceinline__ bool mailbox_wait_sum(const unsigned long long* base, int count,
+                                                 const unsigned long long* base3, int count3, unsigned seq,
+                                                 const int* error, unsigned spin_limit, float& sum, float& sum3) {
+  unsigned spins = 0;
+  for (;;) {
+    unsigned long long word[COUNT + EXTRA];
+#pragma unroll
+    for (int u = 0; u < COUNT; ++u)
+      word[u] = __hip_atomic_load(base + u * STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int u = 0; u < EXTRA; ++u)
+      word[COUNT + u] = __hip_atomic_load(base3 + u * STRIDE3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool ready = true;
+#pragma unroll
+    for (int u = 0; u < COUNT; ++u) ready = ready && (u >= count || (unsigned)(word[u] >> 32) == seq);
+#pragma unroll
+    for (int u = 0; u < EXTRA; ++u) ready = ready && (u >= count3 || (unsigned)(word[COUNT + u] >> 32) == seq);
+    if (ready) {
+#pragma unroll
+      for (int u = 0; u < COUNT; ++u) sum += (u < count) ? __uint_as_float((unsigned)word[u]) : 0.0f;
+#pragma unroll
+      for (int u = 0; u < EXTRA; ++u) sum3 += (u < count3) ? __uint_as_float((unsigned)word[COUNT + u]) : 0.0f;
+      return true;
+    }
+    ++spins;
+    if (spins > spin_limit) return false;
+    if ((spins & 63u) == 0 && __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
 // Householder scalars of a column with leading entry alpha and squared norm x2 of the rest.
 // A column whose squared norm is at most `floor2` is left alone (tau = 0): see kQrNegligible.
 struct Reflector {
@@ -276,6 +313,27 @@ __device__ __forceinline__ Reflector make_reflector(float alpha, float x2, float
     h.tau = (h.beta - alpha) / h.beta;
     h.scale = 1.0f / (alpha - h.beta);
   }
+  return h;
+}
+
+// The same scalars without a division or a correctly rounded square root on the critical path:
+// with r = 1/sqrt(alpha^2 + x2) (hardware estimate plus one Newton step), tau = (beta - alpha)/beta
+// = 1 + |alpha| r and scale = 1/(alpha - beta) = sign(alpha)/(|alpha| + norm) (reciprocal estimate
+// plus one Newton step); each is within about one unit in the last place of the exact value.  Norms
+// whose squares leave the comfortable part of the exponent range take the function above.
+__device__ __forceinline__ Reflector make_reflector_fast(float alpha, float x2, float floor2) {
+  const float nrm2 = alpha * alpha + x2;
+  if (__builtin_expect(!(nrm2 > 1e-30f && nrm2 < 1e30f), 0)) return make_reflector(alpha, x2, floor2);
+  const bool valid = x2 > 0.0f && nrm2 > floor2;
+  float r = __builtin_amdgcn_rsqf(nrm2);
+  r = r * (1.5f - 0.5f * nrm2 * r * r);
+  const float nrm = nrm2 * r, absa = fabsf(alpha), den = absa + nrm;
+  float inv = __builtin_amdgcn_rcpf(den);
+  inv = inv * (2.0f - den * inv);
+  Reflector h;
+  h.beta = valid ? ((alpha >= 0.0f) ? -nrm : nrm) : alpha;
+  h.tau = valid ? 1.0f + absa * r : 0.0f;
+  h.scale = valid ? ((alpha >= 0.0f) ? inv : -inv) : 0.0f;
   return h;
 }
 
@@ -545,6 +603,297 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
     // No barrier here: the shared arrays of the next round's first phase (s_wave, s_piv_out) were
     // last read before the barrier that follows the mailbox phase, and the arrays read above are
     // rewritten only behind the next such barrier, which every wavefront reaches after this point.
+  }
+}
+
+// ---- whole panel per exchange -----------------------------------------------------------------
+// The same compressed problem as above with a round that covers every remaining column of the
+// panel.  The explicit part is the panel's 32 x 32 top block (rows p .. p+31, all owned by the first
+// 32 threads of workgroup 0); everything below it is hidden and enters only through its 32 x 32
+// Gram matrix, which a wavefront computes on the matrix cores: its 64 rows go through LDS once to
+// get from "lane = row" to the operand layout "lane = (row parity, column)", then 32
+// v_mfma_f32_32x32x2 instructions (operand a = operand b) accumulate X^T X.  The workgroups exchange
+// the upper triangle of that matrix (528 words) and the top block (1024 words) once, every
+// workgroup runs all Householder steps of the panel on [top block ; Gram] with the same guard as
+// above (a round ends before a column whose corrected norm has lost three quarters of its terms'
+// size, and that column opens a new round with a freshly computed Gram matrix), and then applies
+// the accepted reflectors to its rows.
+constexpr int kQrGramWords = kQrNb * (kQrNb + 1) / 2;
+
+// Entry `idx` of the packed upper triangle -> (i, k), i <= k.  Rows i and 31 - i together have 33
+// entries, so the triangle is 16 row pairs of 33.
+__device__ __forceinline__ void gram_unpack_index(int idx, int& i, int& k) {
+  const int pair = idx / (kQrNb + 1), off = idx - pair * (kQrNb + 1);
+  if (off < kQrNb - pair) {
+    i = pair;
+    k = pair + off;
+  } else {
+    i = kQrNb - 1 - pair;
+    k = i + (off - (kQrNb - pair));
+  }
+}
+
+// Mailbox layout of the Gram values: nine chunks of 64 values, inside a chunk one 64-word row per
+// workgroup, so that the words one thread sums (one value, all workgroups) lie 512 bytes apart.
+constexpr int kQrGramChunks = (kQrGramWords + 63) / 64;
+constexpr int kQrGramMailWords = kQrGramChunks * 64;  // per workgroup
+__device__ __forceinline__ size_t gram_mail_offset(int idx, int wg) {
+  return ((size_t)(idx >> 6) * kQrPersistentMaxWg + wg) * 64 + (idx & 63);
+}
+
+template <int T0, int T1, class F>
+__device__ __forceinline__ void static_for_by4(F&& f) {
+  if constexpr (T0 < T1) {
+    f(std::integral_constant<int, T0>{});
+    static_for_by4<T0 + 4, T1>(f);
+  }
+}
+
+template <int T0, int T1, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (T0 < T1) {
+    f(std::integral_constant<int, T0>{});
+    static_for<T0 + 1, T1>(f);
+  }
+}
+
+__global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ A, int64_t lda, int n, int p, int pe,
+                                                            unsigned long long* part, unsigned long long* piv,
+                                                            float* __restrict__ tau, unsigned seq_base, int* error,
+                                                            int nwg, unsigned spin_limit, float* __restrict__ vout,
+                                                            int64_t ldv, int vrow0) {
+  using T = float;
+  constexpr int NB = kQrNb, GW = kQrGramWords, XS = NB + 1;
+  static_assert(GW == 512 + 16, "the exchange below splits the Gram values as 2 x 256 + 16");
+  __shared__ T s_x[4][64 * XS];  // a wavefront's rows on their way to the MFMA layout, then its Gram matrix
+  __shared__ T s_tot[NB * NB];   // s_tot[i * NB + k] = G[i][k], both triangles
+  __shared__ T s_piv[NB * NB];   // s_piv[q * NB + k] = entry k of row p + q
+  __shared__ T s_tc[NB][NB];
+  __shared__ T s_scal[NB][2];    // scale, tau of the panel's reflectors
+  __shared__ T s_l3[16][16];     // partial sums of the last 16 Gram values, [value][workgroup residue]
+  __shared__ T s_seen;           // largest squared column norm of this panel so far
+  __shared__ int s_done;
+  __shared__ int s_fail;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wg = blockIdx.x;
+  const int r = p + wg * 256 + tid;
+  const int nbw = pe - p;
+  const bool live = r < n;
+  const bool hidden = live && wg * 256 + tid >= NB;
+  if (tid == 0) {
+    s_fail = 0;
+    s_seen = T(0);
+  }
+  if (wg == 0) {
+    for (int t = tid; t < (p - vrow0) * nbw; t += 256) vout[t % (p - vrow0) + (int64_t)(t / (p - vrow0)) * ldv] = T(0);
+  }
+
+  T a[NB];  // a[k] = A[r, p + k]
+#pragma unroll
+  for (int k = 0; k < NB; ++k) a[k] = (live && k < nbw) ? A[r + (int64_t)(p + k) * lda] : T(0);
+
+  int c = 0;  // finished columns
+  for (unsigned round = 0; c < nbw; ++round) {
+    const unsigned seq = seq_base + round + 1u;
+    unsigned long long* part_c = part + (size_t)(round & 1) * kQrPersistentMaxWg * kQrGramMailWords;
+    unsigned long long* piv_c = piv + (round & 1) * NB * NB;
+    // the top block first: it is on its way while the Gram matrix is being computed
+    if (wg == 0 && tid < NB) {
+#pragma unroll
+      for (int k = 0; k < NB; ++k)
+        __hip_atomic_store(piv_c + tid * NB + k, mailbox_pack(live ? a[k] : T(0), seq), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // Gram matrix of this wavefront's hidden rows (finished columns ride along; nobody reads them)
+    {
+      T* xs = s_x[wave];
+#pragma unroll
+      for (int k = 0; k < NB; ++k) xs[lane * XS + k] = hidden ? a[k] : T(0);
+      __syncthreads();
+      Mfma<T>::Acc acc = {}, acc_odd = {};  // two chains, so that an instruction need not wait for the one before it
+#pragma unroll
+      for (int s = 0; s < 32; s += 2) {
+        const T x0 = xs[(2 * s + (lane >> 5)) * XS + (lane & 31)];
+        const T x1 = xs[(2 * s + 2 + (lane >> 5)) * XS + (lane & 31)];
+        acc = Mfma<T>::mma(x0, x0, acc);
+        acc_odd = Mfma<T>::mma(x1, x1, acc_odd);
+      }
+      acc += acc_odd;
+      // (a wavefront's LDS accesses complete in order: its reads above are done before these writes)
+#pragma unroll
+      for (int v = 0; v < Mfma<T>::NACC; ++v) xs[Mfma<T>::acc_row(v, lane) * NB + (lane & 31)] = acc[v];
+    }
+    __syncthreads();
+    for (int idx = tid; idx < GW; idx += 256) {
+      int i, k;
+      gram_unpack_index(idx, i, k);
+      const int e = i * NB + k;
+      const T sum = (s_x[0][e] + s_x[1][e]) + (s_x[2][e] + s_x[3][e]);
+      __hip_atomic_store(part_c + gram_mail_offset(idx, wg), mailbox_pack(sum, seq), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+    {
+      // Fixed-order sums over the workgroups.  Thread tid takes the values tid and tid + 256 over all
+      // workgroups (48 loads in flight, so one trip each up to 48 workgroups); the 16 values from 512
+      // on are split sixteen ways over the workgroups (thread tid: value 512 + tid % 16, workgroups
+      // tid / 16, tid / 16 + 16, ...) and ride along with the second trip.
+      bool ok = true;
+      constexpr int L3 = kQrPersistentMaxWg / 16, BATCH = 48;  // BATCH * 64 = the spare words behind the buffer
+      T sum[2] = {T(0), T(0)}, sum3 = T(0);
+      const unsigned long long* base3 = part_c + gram_mail_offset(512 + (tid & 15), tid >> 4);
+      const int count3 = (nwg - (tid >> 4) + 15) >> 4;  // workgroups tid / 16, tid / 16 + 16, ... below nwg
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int idx = tid + 256 * half;
+        for (int w0 = 0; w0 < nwg && ok; w0 += BATCH) {
+          // (the last batch may reach past workgroup 127: the buffer has BATCH spare rows)
+          const unsigned long long* base = part_c + gram_mail_offset(idx, w0);
+          T unused = T(0);
+          if (half == 1 && w0 == 0)
+            ok = mailbox_wait_sum<BATCH, 64, L3, 16 * 64>(base, nwg - w0, base3, count3, seq, error, spin_limit, sum[half],
+                                                          sum3);
+          else
+            ok = mailbox_wait_sum<BATCH, 64, 0, 1>(base, nwg - w0, base, 0, seq, error, spin_limit, sum[half], unused);
+        }
+        int i, k;
+        gram_unpack_index(idx, i, k);
+        s_tot[i * NB + k] = sum[half];
+        s_tot[k * NB + i] = sum[half];
+      }
+      s_l3[tid & 15][tid >> 4] = sum3;
+      if (ok) {
+        const unsigned long long* slot[4];
+        const bool used[4] = {true, true, true, true};
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) slot[u] = piv_c + tid + 256 * u;
+        ok = mailbox_wait<4>(slot, used, seq, error, spin_limit, v);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s_piv[tid + 256 * u] = v[u];
+      }
+      if (!ok) {
+        __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_fail = 1;
+      }
+    }
+    __syncthreads();
+    if (s_fail) return;
+    if (tid < 16) {
+      T total = T(0);
+#pragma unroll
+      for (int u = 0; u < 16; ++u) total += s_l3[tid][u];
+      int i, k;
+      gram_unpack_index(512 + tid, i, k);
+      s_tot[i * NB + k] = total;
+      s_tot[k * NB + i] = total;
+    }
+    __syncthreads();
+    if (tid < NB) {
+      // lane k owns column k of the top block (pv) and of G (g)
+      const int k = tid;
+      T pv[NB], g[NB];
+#pragma unroll
+      for (int q = 0; q < NB; ++q) {
+        pv[q] = s_piv[q * NB + k];
+        g[q] = s_tot[q * NB + k];
+      }
+      T size_diag = fabsf(s_tot[k * NB + k]);  // size of the terms G[k][k] is made of
+      T seen = s_seen;
+      int done = c;
+      bool open = true;
+      // Straight-line code per step: once a step has been refused (`open` false) the later steps
+      // still run, on numbers nobody will use - the rows' owners apply only the steps before `done`,
+      // and the next round starts from their rows.
+      static_for<0, NB>([&](auto step) {
+        constexpr int t = decltype(step)::value;
+        if (t >= c && t < nbw) {
+          // e_k = <column t, column k> over the explicit rows below pivot t; lane t's value is the
+          // explicit part of column t's squared norm.  Broadcasts go four at a time so that the
+          // scalar results are not needed by the very next instruction.
+          T e = T(0);
+          static_for_by4<t + 1, NB>([&](auto block) {
+            constexpr int q = decltype(block)::value;
+            T col[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) col[b] = (q + b < NB) ? lane_value<t>(pv[(q + b) & (NB - 1)]) : T(0);
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+              if (q + b < NB) e += col[b] * pv[(q + b) & (NB - 1)];
+          });
+          const T alpha = lane_value<t>(pv[t]);
+          const T hidden2 = lane_value<t>(g[t]);
+          const T x2_explicit = lane_value<t>(e);
+          const T size_t_ = lane_value<t>(size_diag);
+          // (the last column of the matrix has nothing below its pivot: exactly zero, so tau = 0 as in LAPACK)
+          const T x2 = (p + t < n - 1) ? x2_explicit + fmaxf(hidden2, T(0)) : T(0);
+          const bool finite = hidden2 - hidden2 == T(0);
+          open = open && (t == c || (finite && alpha * alpha + x2 >= kQrRoundGuard * size_t_));
+          const Reflector h = make_reflector_fast(alpha, x2, kQrNegligible * seen);
+          seen = open ? fmaxf(seen, alpha * alpha + x2) : seen;  // (what outlives the round must not see a refused step)
+          const T d = g[t] + e;  // <column t, column k> below pivot t
+          const T tc = (k > t) ? h.tau * (pv[t] + h.scale * d) : T(0);
+          s_tc[t][k] = tc;
+          s_scal[t][0] = h.scale;  // (every lane writes the same two numbers)
+          s_scal[t][1] = h.tau;
+          // G[i][k] -= tc_k s G[t][i] + tc_i s G[t][k] - tc_i tc_k s^2 G[t][t]  =  tc_k u_i + tc_i w_k
+          const T w = h.scale * g[t];
+          const T s2gtt = h.scale * h.scale * hidden2;
+          const T u = w - tc * s2gtt;
+          static_for_by4<t + 1, NB>([&](auto block) {
+            constexpr int q = decltype(block)::value;
+            T col[4], ui[4], tci[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              constexpr int last = NB - 1;
+              col[b] = (q + b < NB) ? lane_value<t>(pv[(q + b) & last]) : T(0);
+            }
+            static_for<0, 4>([&](auto bb) {
+              constexpr int b = decltype(bb)::value;
+              if constexpr (q + b < NB) {
+                ui[b] = lane_value<q + b>(u);
+                tci[b] = lane_value<q + b>(tc);
+              }
+            });
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+              if (q + b < NB) {
+                // explicit rows: E[q][k] -= tc_k (E[q][t] s), rounded exactly as the rows' owners do it
+                // further down, so that both hold the same numbers (lane t itself has tc = 0)
+                pv[(q + b) & (NB - 1)] -= tc * (col[b] * h.scale);
+                g[(q + b) & (NB - 1)] = (g[(q + b) & (NB - 1)] - tc * ui[b]) - tci[b] * w;
+              }
+          });
+          size_diag += T(2) * fabsf(tc * w) + fabsf(tc * tc * s2gtt);
+          done = open ? t + 1 : done;
+        }
+      });
+      if (k == 0) {
+        s_done = done;
+        s_seen = seen;
+      }
+    }
+    __syncthreads();
+    const int done = s_done;
+    static_for<0, NB>([&](auto step) {
+      constexpr int t = decltype(step)::value;
+      if (t >= c && t < done) {
+        const T scale = s_scal[t][0];
+        const int jt = p + t;
+        // one instruction stream for the rows below the pivot (v = scaled entry), the pivot row
+        // (v = 1) and the finished rows above it (v = 0)
+        const bool below = r > jt, pivot = r == jt;
+        const T v = below ? a[t] * scale : (pivot ? T(1) : T(0));
+#pragma unroll
+        for (int k = t + 1; k < NB; ++k) a[k] -= s_tc[t][k] * v;
+        if (live && pivot) tau[jt] = s_scal[t][1];
+        if (live) {
+          // clean form in both copies, as in the kernel above
+          A[r + (int64_t)jt * lda] = v;
+          vout[(r - vrow0) + (int64_t)t * ldv] = v;
+        }
+      }
+    });
+    c = done;
   }
 }
 
@@ -952,6 +1301,13 @@ static inline void launch_extract_v(hipStream_t s, const T* A, int64_t lda, int 
 }
 
 // ---- QR driver -------------------------------------------------------------------------------
+// Mailbox words per workgroup and for the pivot rows: the larger of what the two persistent panel
+// kernels use (four columns per round: 4 x 32 and 4 x 32; whole panel: 9 x 64 and 32 x 32).
+constexpr int kQrMailWords = kQrGramMailWords > kQrRoundMax * kQrNb ? kQrGramMailWords : kQrRoundMax * kQrNb;
+constexpr int kQrMailPivotWords = kQrNb * kQrNb;
+constexpr int kQrMailSpareWords = 48 * 64;  // the whole-panel kernel loads rows of 48 workgroups at a time, used or not
+constexpr int kQrWholePanel = kQrNb;  // columns_per_round value that selects qr_panel_gram_kernel
+
 template <typename T>
 struct QrWorkspace {
   BlockReflectorWs<T> br;
@@ -959,8 +1315,8 @@ struct QrWorkspace {
   T* tau;     // n
   T* part;    // 2 x nwg x NB   partials of the launch-per-column fallback
   T* piv;     // 2 x NB
-  unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x kQrRoundMax NB   mailboxes of the persistent panel kernel
-  unsigned long long* mail_piv;   // 2 x kQrRoundMax NB
+  unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x kQrMailWords   mailboxes of the persistent panel kernels
+  unsigned long long* mail_piv;   // 2 x kQrMailPivotWords
   unsigned* sync;  // [1] error flag of the persistent panel kernel
 };
 
@@ -974,8 +1330,8 @@ static inline void qr_workspace_layout(WS& ws, int64_t n, QrWorkspace<T>* out) {
   q.tau = ws.template take<T>((size_t)n);
   q.part = ws.template take<T>((size_t)2 * nwg * kQrNb);
   q.piv = ws.template take<T>(2 * kQrNb);
-  q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * kQrRoundMax * kQrNb);
-  q.mail_piv = ws.template take<unsigned long long>(2 * kQrRoundMax * kQrNb);
+  q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * kQrMailWords + kQrMailSpareWords);
+  q.mail_piv = ws.template take<unsigned long long>(2 * kQrMailPivotWords);
   q.sync = ws.template take<unsigned>(64);
   if (out) *out = q;
 }
@@ -1004,8 +1360,9 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
   unsigned seq_base = 0;
   hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
   {
-    // mail_part and mail_piv are adjacent: one clear covers both (sequence number 0 = "nothing yet")
-    const int words = 2 * (2 * kQrPersistentMaxWg * kQrRoundMax * kQrNb + 2 * kQrRoundMax * kQrNb);
+    // sequence number 0 = "nothing yet"; mail_piv follows mail_part in the workspace, one clear covers both
+    const int words = (int)(reinterpret_cast<unsigned*>(ws.mail_piv + 2 * kQrMailPivotWords) -
+                            reinterpret_cast<unsigned*>(ws.mail_part));
     hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3((words + 255) / 256), dim3(256), 0, s,
                        reinterpret_cast<unsigned*>(ws.mail_part), words);
   }
@@ -1025,7 +1382,12 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       // this panel's reflectors inside the outer block's n x 128 buffer (origin: row P, column P)
       BlockReflectorWs<T> inner = ws.br;
       inner.v = ws.br.v + (p - P) + (int64_t)(p - P) * ldv;
-      if (nwg <= persistent_max_wg) {
+      if (nwg <= persistent_max_wg && columns_per_round == kQrWholePanel) {
+        hipLaunchKernelGGL(qr_panel_gram_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part, ws.mail_piv,
+                           ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
+                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P);
+        seq_base += (unsigned)nbw;
+      } else if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
                            ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
                            ws.br.v + (int64_t)(p - P) * ldv, ldv, P, columns_per_round);

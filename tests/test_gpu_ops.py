@@ -218,7 +218,7 @@ def test_qr_block_reflector_widths(size, device):
 
 
 @pytest.mark.parametrize("kind", ["paired_columns", "graded", "rank_deficient", "repeated_column"])
-@pytest.mark.parametrize("columns_per_round", [1, 2, 3, 4])
+@pytest.mark.parametrize("columns_per_round", [1, 2, 3, 4, 32])
 def test_qr_is_backward_stable_on_hard_matrices(kind, columns_per_round, device):
     """Orthogonality of Q and the backward error of A = Q R on matrices built to hurt a panel that
     derives a column's norm from dot products: neighbouring columns that are nearly parallel,
@@ -240,7 +240,7 @@ def test_qr_is_backward_stable_on_hard_matrices(kind, columns_per_round, device)
         factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
         ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
     finally:
-        _native.call("soapmi_set_option", b"qr_columns_per_round", 4)
+        _native.call("soapmi_set_option", b"qr_columns_per_round", 32)
     q = factor.cpu().double()
     a = matrix.double()
     assert torch.isfinite(q).all()
