@@ -1242,6 +1242,134 @@ __global__ __launch_bounds__(256) void reflector_w2_solve_kernel(const T* __rest
   if (mine) W2[l + (int64_t)c * ldw2] = x;
 }
 
+// In-block update of a 32-column panel in one launch: C (rows x nc, ld ldc) <- C - V X with
+// X = T^T (V^T C) obtained as in reflector_w2_solve_kernel from the split-K slices of V^T [V | C].
+// A workgroup owns 256 rows and kPanelApplyCols columns.  Every workgroup of a column group sums
+// the slices and solves for X itself (the same numbers in the same order everywhere: 12 KB per
+// slice, a forward substitution of 32 steps with one lane per column), which costs less than a
+// launch of its own; the product then runs on the matrix cores with the roles of rows and columns
+// swapped, D[column][row] += (-X)^T[column][k] V^T[k][row], so that the lanes of a wavefront walk
+// down a column of C and of V (coalesced) and X comes out of LDS.
+constexpr int kPanelApplyCols = 64;
+
+__global__ __launch_bounds__(256) void panel_apply_kernel(const float* __restrict__ part, int splits, int64_t slab,
+                                                          int nc, const float* __restrict__ tau,
+                                                          const float* __restrict__ V, int64_t ldv,
+                                                          float* __restrict__ C, int64_t ldc, int rows) {
+  using T = float;
+  constexpr int M = kQrNb, NC = kPanelApplyCols;
+  __shared__ __align__(16) T s_g[M][M];   // s_g[i][l] = (V^T V)[i][l], read for i < l
+  __shared__ T s_w[NC][M + 1];            // s_w[c][i] = (V^T C)[i][c] of this column group
+  __shared__ T s_xn[M][NC];               // s_xn[k][c] = -X[k][c]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col0 = blockIdx.y * NC;
+  // Rows 64 wave .. 64 wave + 63 of the workgroup: two row tiles by two column tiles of 32 x 32.
+  // The tile of C and the rows of V are requested first; they arrive while X is being made.
+  const int64_t row_base = (int64_t)blockIdx.x * 256 + wave * 64;
+  const int jr = lane & 31, half = lane >> 5;
+  Mfma<T>::Acc acc[2][2];
+  T vb[2][M / 2];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int64_t r = row_base + rt * 32 + jr;
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int v = 0; v < Mfma<T>::NACC; ++v) {
+        const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
+        acc[rt][ct][v] = (r < rows && c < nc) ? C[r + (int64_t)c * ldc] : T(0);
+      }
+#pragma unroll
+    for (int ks = 0; ks < M / 2; ++ks) vb[rt][ks] = (r < rows) ? V[r + (int64_t)(2 * ks + half) * ldv] : T(0);
+  }
+  {
+    // fixed-order sums over the slices: four entries of G and eight of W per thread
+    int offset[12];
+    bool inside[12];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = tid + 256 * q;  // row e % 32, column e / 32 of G
+      inside[q] = true;
+      offset[q] = e;
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int e = tid + 256 * q, row = e & 31, c = col0 + (e >> 5);
+      inside[4 + q] = c < nc;
+      offset[4 + q] = inside[4 + q] ? row + (M + c) * M : 0;
+    }
+    T sum[12];
+#pragma unroll
+    for (int q = 0; q < 12; ++q) sum[q] = T(0);
+    int z = 0;
+    for (; z + 4 <= splits; z += 4) {  // four slices' loads in flight
+      T v[4][12];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int q = 0; q < 12; ++q) v[u][q] = part[(int64_t)(z + u) * slab + offset[q]];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int q = 0; q < 12; ++q) sum[q] += v[u][q];
+    }
+    for (; z < splits; ++z) {
+      T v[12];
+#pragma unroll
+      for (int q = 0; q < 12; ++q) v[q] = part[(int64_t)z * slab + offset[q]];
+#pragma unroll
+      for (int q = 0; q < 12; ++q) sum[q] += v[q];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = tid + 256 * q;
+      s_g[e & 31][e >> 5] = sum[q];
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int e = tid + 256 * q;
+      s_w[e >> 5][e & 31] = inside[4 + q] ? sum[4 + q] : T(0);
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // x_i = tau_i (w_i - sum_{l < i} G[l][i] x_l), one lane per column
+    T w[M];
+#pragma unroll
+    for (int i = 0; i < M; ++i) w[i] = s_w[lane][i];
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      const T xi = tau[i] * w[i];
+      s_xn[i][lane] = -xi;
+#pragma unroll
+      for (int l = i + 1; l < M; ++l) w[l] -= s_g[i][l] * xi;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int ks = 0; ks < M / 2; ++ks) {
+    const int k = 2 * ks + half;
+    T a[2];
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) a[ct] = s_xn[k][ct * 32 + jr];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct) acc[rt][ct] = Mfma<T>::mma(a[ct], vb[rt][ks], acc[rt][ct]);
+  }
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      const int64_t r = row_base + rt * 32 + jr;
+#pragma unroll
+      for (int v = 0; v < Mfma<T>::NACC; ++v) {
+        const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
+        if (r < rows && c < nc) C[r + (int64_t)c * ldc] = acc[rt][ct][v];
+      }
+    }
+}
+
 template <typename T>
 static inline int gram_of_v(hipStream_t s, const BlockReflectorWs<T>& ws, int rows, int nbw, int64_t ldv) {
   using Skinny = typename SkinnyTile<T>::type;
@@ -1413,11 +1541,18 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
                                          split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
                                          ws.br.splitk, &slices);
         if (rc) return rc;
-        hipLaunchKernelGGL((reflector_w2_solve_kernel<T>), dim3((unsigned)ceil_div64(nc, kW2SolveCols)), dim3(256), 0, s,
-                           ws.br.splitk, slices, (int64_t)nbw * ncols, nbw, nc, ws.tau + p, ws.br.w2, kBrMax);
-        SOAPMI_LAUNCH_CHECK();
-        rc = gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), inner.v, ldv, ws.br.w2, kBrMax, T(1), A + p + (int64_t)pe * lda, lda);
-        if (rc) return rc;
+        if (nbw == NB) {
+          hipLaunchKernelGGL(panel_apply_kernel, dim3((unsigned)ceil_div64(rows, 256), (unsigned)ceil_div64(nc, kPanelApplyCols)),
+                             dim3(256), 0, s, ws.br.splitk, slices, (int64_t)nbw * ncols, nc, ws.tau + p, inner.v, ldv,
+                             A + p + (int64_t)pe * lda, lda, rows);
+          SOAPMI_LAUNCH_CHECK();
+        } else {
+          hipLaunchKernelGGL((reflector_w2_solve_kernel<T>), dim3((unsigned)ceil_div64(nc, kW2SolveCols)), dim3(256), 0, s,
+                             ws.br.splitk, slices, (int64_t)nbw * ncols, nbw, nc, ws.tau + p, ws.br.w2, kBrMax);
+          SOAPMI_LAUNCH_CHECK();
+          rc = gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), inner.v, ldv, ws.br.w2, kBrMax, T(1), A + p + (int64_t)pe * lda, lda);
+          if (rc) return rc;
+        }
       } else if (pe < PE) {
         T* Tin = Tm + (int64_t)(p - P) * (OB + 1);  // diagonal block of the outer factor
         launch_extract_v<T>(s, A, lda, rows, p, p, nbw, inner.v, ldv);
