@@ -641,6 +641,10 @@ __device__ __forceinline__ size_t gram_mail_offset(int idx, int wg) {
   return ((size_t)(idx >> 6) * kQrPersistentMaxWg + wg) * 64 + (idx & 63);
 }
 
+// Workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global load
+// and store of the wavefront, which would expose the latency of loads issued ahead on purpose.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <int T0, int T1, class F>
 __device__ __forceinline__ void static_for_by4(F&& f) {
   if constexpr (T0 < T1) {
@@ -661,11 +665,13 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
                                                             unsigned long long* part, unsigned long long* piv,
                                                             float* __restrict__ tau, unsigned seq_base, int* error,
                                                             int nwg, unsigned spin_limit, float* __restrict__ vout,
-                                                            int64_t ldv, int vrow0) {
+                                                            int64_t ldv, int vrow0, float* __restrict__ slices, int nc,
+                                                            int64_t slab) {
   using T = float;
   constexpr int NB = kQrNb, GW = kQrGramWords, XS = NB + 1;
   static_assert(GW == 512 + 16, "the exchange below splits the Gram values as 2 x 256 + 16");
   __shared__ T s_x[4][64 * XS];  // a wavefront's rows on their way to the MFMA layout, then its Gram matrix
+  __shared__ T s_sum[4][NB * NB];  // the wavefronts' parts of a 32 x 32 block of V^T [V | C]
   __shared__ T s_tot[NB * NB];   // s_tot[i * NB + k] = G[i][k], both triangles
   __shared__ T s_piv[NB * NB];   // s_piv[q * NB + k] = entry k of row p + q
   __shared__ T s_tc[NB][NB];
@@ -891,9 +897,85 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
           A[r + (int64_t)jt * lda] = v;
           vout[(r - vrow0) + (int64_t)t * ldv] = v;
         }
+        a[t] = v;  // the finished column's register now holds this row of V (nothing reads it before the end)
       }
     });
     c = done;
+  }
+  if (slices == nullptr) return;
+  // ---- this workgroup's slice of V^T [V | C] ------------------------------------------------------
+  // C = the nc columns behind the panel (the rest of the outer block), V = the panel's reflectors,
+  // both over this workgroup's 256 rows.  The in-block update needs the sums of these slices over
+  // the workgroups; computing them here saves a launch that would read V and C again.  A wavefront
+  // multiplies its own 64 rows: V goes through LDS once into the "b" operand layout (32 registers),
+  // each 32-column block of C is loaded row per lane (256 contiguous bytes per instruction), passed
+  // through the same LDS area into the "a" layout and multiplied with 32 v_mfma_f32_32x32x2; the four
+  // wavefronts' results are added through LDS in a fixed order.  Block 0 is V^T V.
+  // Slice layout: element (i, j) of the 32 x (32 + nc) matrix at slices[wg * slab + i + 32 * j].
+  {
+    T* xs = s_x[wave];
+    const int half = lane >> 5, l31 = lane & 31;
+    const int blocks = 1 + (nc + NB - 1) / NB;
+    // Loads are unconditional on clamped addresses (a row past the end reads the last row, a column
+    // past the end the last column): such rows have V = 0 and such columns are not stored.  The
+    // column's base address is the same for all lanes, the row a 32-bit index.
+    const int rr = live ? r : n - 1;
+    T cur[NB];
+    auto load_block = [&](int c0) {
+      const T* base = A + (int64_t)(pe + c0) * lda;
+      if (c0 + NB <= nc) {
+#pragma unroll
+        for (int k = 0; k < NB; ++k) cur[k] = base[(int64_t)k * lda + rr];
+      } else {
+#pragma unroll
+        for (int k = 0; k < NB; ++k) cur[k] = base[(int64_t)min(k, nc - 1 - c0) * lda + rr];
+      }
+    };
+    if (blocks > 1) load_block(0);  // on its way while V is staged and V^T V computed
+#pragma unroll
+    for (int k = 0; k < NB; ++k) xs[lane * XS + k] = a[k];
+    T vb[NB];
+#pragma unroll
+    for (int s = 0; s < NB; ++s) vb[s] = xs[(2 * s + half) * XS + l31];
+    auto emit = [&](int jb, const Mfma<T>::Acc& acc) {
+#pragma unroll
+      for (int v = 0; v < Mfma<T>::NACC; ++v) s_sum[wave][Mfma<T>::acc_row(v, lane) * NB + l31] = acc[v];
+      lds_barrier();
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int e = tid + 256 * q;  // i = e % 32, j = 32 jb + e / 32
+        if (jb * NB + (e >> 5) < NB + nc)
+          slices[(int64_t)wg * slab + jb * (NB * NB) + e] = (s_sum[0][e] + s_sum[1][e]) + (s_sum[2][e] + s_sum[3][e]);
+      }
+      lds_barrier();
+    };
+    {
+      Mfma<T>::Acc acc = {}, acc_odd = {};
+#pragma unroll
+      for (int s = 0; s < NB; s += 2) {
+        acc = Mfma<T>::mma(vb[s], vb[s], acc);
+        acc_odd = Mfma<T>::mma(vb[s + 1], vb[s + 1], acc_odd);
+      }
+      acc += acc_odd;
+      emit(0, acc);
+    }
+    for (int jb = 1; jb < blocks; ++jb) {
+      // (a wavefront's LDS accesses complete in order: the reads of the block before are done)
+#pragma unroll
+      for (int k = 0; k < NB; ++k) xs[lane * XS + k] = cur[k];
+      if (jb + 1 < blocks) load_block(jb * NB);  // the next block's loads are in flight during this block's products
+      T x[NB];
+#pragma unroll
+      for (int s = 0; s < NB; ++s) x[s] = xs[(2 * s + half) * XS + l31];
+      Mfma<T>::Acc acc = {}, acc_odd = {};
+#pragma unroll
+      for (int s = 0; s < NB; s += 2) {
+        acc = Mfma<T>::mma(x[s], vb[s], acc);
+        acc_odd = Mfma<T>::mma(x[s + 1], vb[s + 1], acc_odd);
+      }
+      acc += acc_odd;
+      emit(jb, acc);
+    }
   }
 }
 
@@ -1510,10 +1592,14 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       // this panel's reflectors inside the outer block's n x 128 buffer (origin: row P, column P)
       BlockReflectorWs<T> inner = ws.br;
       inner.v = ws.br.v + (p - P) + (int64_t)(p - P) * ldv;
+      bool slices_by_panel = false;
       if (nwg <= persistent_max_wg && columns_per_round == kQrWholePanel) {
+        // (a full panel with columns of the outer block behind it also leaves its slices of V^T [V | C])
+        slices_by_panel = pe < PE && nbw == NB;
         hipLaunchKernelGGL(qr_panel_gram_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part, ws.mail_piv,
                            ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
-                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P);
+                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, slices_by_panel ? ws.br.splitk : nullptr, PE - pe,
+                           (int64_t)NB * (PE - p));
         seq_base += (unsigned)nbw;
       } else if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
@@ -1536,11 +1622,13 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
         // diagonal blocks of the outer factor are all built after the block's last panel.
         using Skinny = typename SkinnyTile<T>::type;
         const int ncols = PE - p, nc = PE - pe;
-        int slices = 1;
-        rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, ncols, rows, inner.v, ldv, A + p + (int64_t)p * lda, lda,
-                                         split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
-                                         ws.br.splitk, &slices);
-        if (rc) return rc;
+        int slices = nwg;
+        if (!slices_by_panel) {
+          rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, ncols, rows, inner.v, ldv, A + p + (int64_t)p * lda, lda,
+                                           split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
+                                           ws.br.splitk, &slices);
+          if (rc) return rc;
+        }
         if (nbw == NB) {
           hipLaunchKernelGGL(panel_apply_kernel, dim3((unsigned)ceil_div64(rows, 256), (unsigned)ceil_div64(nc, kPanelApplyCols)),
                              dim3(256), 0, s, ws.br.splitk, slices, (int64_t)nbw * ncols, nc, ws.tau + p, inner.v, ldv,
