@@ -114,10 +114,14 @@ struct EpiAdam {
 };
 
 // ---- kernel ------------------------------------------------------------------------------
-template <typename T, int BM_, int BN_, int BK_, int WM_, int WN_>
+// KS_ > 1: KS_ groups of WM_ x WN_ wavefronts share a tile; each group multiplies its own part of
+// every K-slab and the groups' accumulators are added through LDS before the epilogue.  For tiles
+// so small that a wavefront holds a single accumulator block, this puts two wavefronts on every
+// SIMD, so that one's LDS waits hide behind the other's matrix instructions.
+template <typename T, int BM_, int BN_, int BK_, int WM_, int WN_, int KS_ = 1>
 struct GemmTile {
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
-  static constexpr int NT = 64 * WM * WN;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, KS = KS_;
+  static constexpr int NT = 64 * WM * WN * KS;
   static constexpr int MI = Mfma<T>::MI, KI = Mfma<T>::KI;
   static constexpr int TM = BM / WM / MI, TN = BN / WN / MI;
   static constexpr int VW = Vec16<T>::W;
@@ -125,7 +129,9 @@ struct GemmTile {
   static constexpr int SA = BM + PAD, SB = BN + PAD;
   static constexpr int NVA = BK * BM / VW / NT, NVB = BK * BN / VW / NT;
   static_assert(BM % (WM * MI) == 0 && BN % (WN * MI) == 0, "wave tiling");
-  static_assert(BK % KI == 0 && BK % VW == 0, "k tiling");
+  static_assert(BK % (KI * KS) == 0 && BK % VW == 0, "k tiling");
+  static_assert(KS == 1 || (KS - 1) * TM * TN * Mfma<T>::NACC * (NT / KS) <= 2 * BK * (BM + PAD + BN + PAD),
+                "the groups' accumulators are exchanged through the operands' LDS buffers");
   static_assert((BK * BM / VW) % NT == 0 && (BK * BN / VW) % NT == 0, "loader tiling");
 };
 
@@ -264,8 +270,9 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
   constexpr bool FAST = MODE >= 0;
   constexpr bool AXC = (MODE & 1) != 0, BXC = (MODE & 2) != 0;
 
-  __shared__ __attribute__((aligned(16))) T As[2][BK * SA];
-  __shared__ __attribute__((aligned(16))) T Bs[2][BK * SB];
+  __shared__ __attribute__((aligned(16))) T smem[2 * BK * SA + 2 * BK * SB];
+  T(*As)[BK * SA] = reinterpret_cast<T(*)[BK * SA]>(smem);
+  T(*Bs)[BK * SB] = reinterpret_cast<T(*)[BK * SB]>(smem + 2 * BK * SA);
 
   // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each XCD one
   // contiguous range of tiles so that neighbouring tiles share its L2.
@@ -294,8 +301,10 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wm0 = (wave % Cfg::WM) * (TM * MI);
-  const int wn0 = (wave / Cfg::WM) * (TN * MI);
+  constexpr int KS = Cfg::KS, KSTEPS = BK / KI / KS;  // k steps of a slab per wavefront group
+  const int wave_mn = wave % (Cfg::WM * Cfg::WN), wave_k = wave / (Cfg::WM * Cfg::WN);
+  const int wm0 = (wave_mn % Cfg::WM) * (TM * MI);
+  const int wn0 = (wave_mn / Cfg::WM) * (TN * MI);
 
   typename MF::Acc acc[TM][TN];
 #pragma unroll
@@ -343,9 +352,9 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
     const T* as = As[buf];
     const T* bs = Bs[buf];
 #pragma unroll
-    for (int kk = 0; kk < BK / KI; ++kk) {
+    for (int kk = 0; kk < KSTEPS; ++kk) {
       T fm[TM], fn[TN];
-      const int kr = kk * KI + krow;
+      const int kr = (wave_k * KSTEPS + kk) * KI + krow;
 #pragma unroll
       for (int i = 0; i < TM; ++i) fm[i] = as[kr * SA + wm0 + i * MI + idx];
 #pragma unroll
@@ -360,6 +369,33 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
       store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[buf ^ 1], rb, b_xc, tid);
     }
     __syncthreads();
+  }
+
+  if constexpr (KS > 1) {
+    // (the loop's last barrier is behind every read of the operand buffers)
+    constexpr int GT = NT / KS;  // threads of a group
+    T* red = smem;
+    const int t_in = tid % GT;
+    if (wave_k > 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < MF::NACC; ++r)
+            red[(((wave_k - 1) * TM + i) * TN + j) * MF::NACC * GT + r * GT + t_in] = acc[i][j][r];
+    }
+    __syncthreads();
+    if (wave_k > 0) return;
+#pragma unroll
+    for (int g = 1; g < KS; ++g)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < MF::NACC; ++r)
+            acc[i][j][r] += red[(((g - 1) * TM + i) * TN + j) * MF::NACC * GT + r * GT + t_in];
   }
 
 #pragma unroll
@@ -468,6 +504,12 @@ struct DefaultTile<double> {
 template <typename T>
 struct SmallTile {
   using type = GemmTile<T, 64, 64, 16, 2, 2>;
+};
+// fp32: a wavefront's share of the tile is a single 32 x 32 accumulator block, so two groups of four
+// wavefronts split each (32 deep) K-slab between them.
+template <>
+struct SmallTile<float> {
+  using type = GemmTile<float, 64, 64, 32, 2, 2, 2>;
 };
 
 // True if an M x N output has so few default tiles that the 256 CUs are badly filled: at most half
