@@ -695,8 +695,15 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
   }
 
   T a[NB];  // a[k] = A[r, p + k]
+  {
+    // (unconditional loads on clamped addresses, zeroed afterwards: tested loads compile to a branch each)
+    const T* arow = A + (live ? r : n - 1) + (int64_t)p * lda;
 #pragma unroll
-  for (int k = 0; k < NB; ++k) a[k] = (live && k < nbw) ? A[r + (int64_t)(p + k) * lda] : T(0);
+    for (int k = 0; k < NB; ++k) {
+      const T x = arow[(int64_t)min(k, nbw - 1) * lda];
+      a[k] = (live && k < nbw) ? x : T(0);
+    }
+  }
 
   int c = 0;  // finished columns
   for (unsigned round = 0; c < nbw; ++round) {
@@ -1351,81 +1358,112 @@ __global__ __launch_bounds__(256) void panel_apply_kernel(const float* __restric
   const int jr = lane & 31, half = lane >> 5;
   Mfma<T>::Acc acc[2][2];
   T vb[2][M / 2];
+  // (loads are unconditional: a row past the end reads the last row and is not stored; a column group
+  // that reaches past the last column takes the slower, tested loads)
+  const bool full_cols = col0 + NC <= nc;
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
-    const int64_t r = row_base + rt * 32 + jr;
+    const int64_t r = min(row_base + rt * 32 + jr, (int64_t)rows - 1);
+    const T* vrow = V + r + (int64_t)half * ldv;
+    const T* crow = C + r + (int64_t)(col0 + 4 * half) * ldc;
+    if (full_cols) {
 #pragma unroll
-    for (int ct = 0; ct < 2; ++ct)
+      for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-      for (int v = 0; v < Mfma<T>::NACC; ++v) {
-        const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
-        acc[rt][ct][v] = (r < rows && c < nc) ? C[r + (int64_t)c * ldc] : T(0);
-      }
+        for (int v = 0; v < Mfma<T>::NACC; ++v)
+          acc[rt][ct][v] = crow[(int64_t)(ct * 32 + 8 * (v >> 2) + (v & 3)) * ldc];  // column col0 + ct * 32 + acc_row(v, lane)
+    } else {
 #pragma unroll
-    for (int ks = 0; ks < M / 2; ++ks) vb[rt][ks] = (r < rows) ? V[r + (int64_t)(2 * ks + half) * ldv] : T(0);
+      for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+        for (int v = 0; v < Mfma<T>::NACC; ++v) {
+          const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
+          acc[rt][ct][v] = (c < nc) ? C[r + (int64_t)c * ldc] : T(0);
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < M / 2; ++ks) vb[rt][ks] = vrow[(int64_t)(2 * ks) * ldv];
   }
   {
-    // fixed-order sums over the slices: four entries of G and eight of W per thread
-    int offset[12];
-    bool inside[12];
+    // Fixed-order sums over the slices, 16 bytes per load: thread tid takes entries 4 tid .. 4 tid + 3
+    // of G (four rows of one column) and two such quadruples of this column group's part of W, which
+    // is one contiguous run of 64 x 32 words in a slice.
+    const int eg = 4 * tid;
+    int offset[3];
+    bool inside[3];
+    offset[0] = eg;
+    inside[0] = true;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int e = tid + 256 * q;  // row e % 32, column e / 32 of G
-      inside[q] = true;
-      offset[q] = e;
+    for (int q = 0; q < 2; ++q) {
+      const int e = eg + 1024 * q, c = col0 + (e >> 5);
+      inside[1 + q] = c < nc;
+      offset[1 + q] = inside[1 + q] ? (M + col0) * M + e : 0;
     }
+    float4 sum[3];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const int e = tid + 256 * q, row = e & 31, c = col0 + (e >> 5);
-      inside[4 + q] = c < nc;
-      offset[4 + q] = inside[4 + q] ? row + (M + c) * M : 0;
-    }
-    T sum[12];
-#pragma unroll
-    for (int q = 0; q < 12; ++q) sum[q] = T(0);
+    for (int q = 0; q < 3; ++q) sum[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto add4 = [](float4& acc4, const float4& x) {
+      acc4.x += x.x;
+      acc4.y += x.y;
+      acc4.z += x.z;
+      acc4.w += x.w;
+    };
     int z = 0;
-    for (; z + 4 <= splits; z += 4) {  // four slices' loads in flight
-      T v[4][12];
+    for (; z + 8 <= splits; z += 8) {  // eight slices' loads in flight
+      float4 v[8][3];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 8; ++u)
 #pragma unroll
-        for (int q = 0; q < 12; ++q) v[u][q] = part[(int64_t)(z + u) * slab + offset[q]];
+        for (int q = 0; q < 3; ++q) v[u][q] = *reinterpret_cast<const float4*>(part + (int64_t)(z + u) * slab + offset[q]);
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 8; ++u)
 #pragma unroll
-        for (int q = 0; q < 12; ++q) sum[q] += v[u][q];
+        for (int q = 0; q < 3; ++q) add4(sum[q], v[u][q]);
     }
     for (; z < splits; ++z) {
-      T v[12];
+      float4 v[3];
 #pragma unroll
-      for (int q = 0; q < 12; ++q) v[q] = part[(int64_t)z * slab + offset[q]];
+      for (int q = 0; q < 3; ++q) v[q] = *reinterpret_cast<const float4*>(part + (int64_t)z * slab + offset[q]);
 #pragma unroll
-      for (int q = 0; q < 12; ++q) sum[q] += v[q];
+      for (int q = 0; q < 3; ++q) add4(sum[q], v[q]);
+    }
+    {
+      const int row = eg & 31, col = eg >> 5;
+      s_g[row][col] = sum[0].x;
+      s_g[row + 1][col] = sum[0].y;
+      s_g[row + 2][col] = sum[0].z;
+      s_g[row + 3][col] = sum[0].w;
     }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int e = tid + 256 * q;
-      s_g[e & 31][e >> 5] = sum[q];
-    }
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const int e = tid + 256 * q;
-      s_w[e >> 5][e & 31] = inside[4 + q] ? sum[4 + q] : T(0);
+    for (int q = 0; q < 2; ++q) {
+      const int e = eg + 1024 * q, row = e & 31, col = e >> 5;
+      const float4 t = inside[1 + q] ? sum[1 + q] : make_float4(0.f, 0.f, 0.f, 0.f);
+      s_w[col][row] = t.x;
+      s_w[col][row + 1] = t.y;
+      s_w[col][row + 2] = t.z;
+      s_w[col][row + 3] = t.w;
     }
   }
   __syncthreads();
   if (wave == 0) {
-    // x_i = tau_i (w_i - sum_{l < i} G[l][i] x_l), one lane per column
-    T w[M];
-#pragma unroll
-    for (int i = 0; i < M; ++i) w[i] = s_w[lane][i];
+    // x_i = tau_i (w_i - sum_{l < i} G[l][i] x_l), one lane per column.  G comes out of registers
+    // (lane l holds column l of G; an entry is read across lanes into a scalar): with the entries
+    // in LDS every pair of multiply-adds waited for its own LDS read.
+    T w[M], gcol[M];
 #pragma unroll
     for (int i = 0; i < M; ++i) {
+      w[i] = s_w[lane][i];
+      gcol[i] = s_g[i][lane & 31];
+    }
+    static_for<0, M>([&](auto step) {
+      constexpr int i = decltype(step)::value;
       const T xi = tau[i] * w[i];
       s_xn[i][lane] = -xi;
-#pragma unroll
-      for (int l = i + 1; l < M; ++l) w[l] -= s_g[i][l] * xi;
-    }
+      static_for<i + 1, M>([&](auto col) {
+        constexpr int l = decltype(col)::value;
+        w[l] -= lane_value<l>(gcol[i]) * xi;
+      });
+    });
   }
   __syncthreads();
 #pragma unroll
