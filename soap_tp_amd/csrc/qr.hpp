@@ -4,13 +4,17 @@
 //
 // Panel (NB = 32 columns): a workgroup owns 256 rows, one per thread, and keeps its row of the
 // panel in registers.  Normally the whole panel runs in one persistent launch whose workgroups
-// exchange partial dot products through device memory, up to four columns per exchange
-// (qr_panel_persistent_kernel); beyond kQrPersistentMaxWg workgroups it runs one launch per column
-// (qr_panel_step_kernel: launch j applies reflector j, whose dot products with the remaining
-// panel columns were reduced by launch j-1, and in the same pass reduces the dot products reflector
-// j+1 needs).  Reductions are a 32-value butterfly over the wavefront, then a fixed-order sum over
-// workgroups: no atomics on data, so results do not depend on scheduling.
-// Trailing matrix and Q formation: compact-WY block reflectors on the MFMA GEMM.
+// exchange, once, the 32 x 32 Gram matrix of their rows (computed on the matrix cores) through
+// device memory; every workgroup then runs the panel's Householder steps on [top block ; Gram],
+// applies the reflectors to its rows and leaves its slice of V^T [V | C] for the update of the
+// rest of the outer block (qr_panel_gram_kernel).  qr_panel_persistent_kernel is the same launch
+// with one to four columns per exchange and partial dot products instead of a Gram matrix; beyond
+// kQrPersistentMaxWg workgroups the panel runs one launch per column (qr_panel_step_kernel: launch
+// j applies reflector j, whose dot products with the remaining panel columns were reduced by launch
+// j-1, and in the same pass reduces the dot products reflector j+1 needs).  Sums over workgroups
+// have a fixed order and use no atomics on data, so results do not depend on scheduling.
+// In-block update: one launch per panel (panel_apply_kernel).  Trailing matrix and Q formation:
+// compact-WY block reflectors on the MFMA GEMM.
 #pragma once
 #include <type_traits>
 
