@@ -649,6 +649,19 @@ __device__ __forceinline__ size_t gram_mail_offset(int idx, int wg) {
 // and store of the wavefront, which would expose the latency of loads issued ahead on purpose.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Value of `v` in lane LANE of the caller's half of the wavefront (lanes 0..31 or 32..63), in every
+// lane of that half.  Only issues the instruction: the result may be used after lds_wait_all() and,
+// so that the compiler keeps the use there, keep_behind_wait() on it.
+template <int LANE>
+__device__ __forceinline__ float half_broadcast_issue(float v) {
+  float r;
+  asm volatile("ds_swizzle_b32 %0, %1 offset:%2" : "=v"(r) : "v"(v), "n"(LANE << 5));  // and 0, or LANE, xor 0
+  return r;
+}
+__device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void keep_behind_wait(float& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void keep_behind_wait(int& v) { asm volatile("" : "+v"(v)); }
+
 template <int T0, int T1, class F>
 __device__ __forceinline__ void static_for_by4(F&& f) {
   if constexpr (T0 < T1) {
@@ -805,16 +818,21 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       s_tot[k * NB + i] = total;
     }
     __syncthreads();
-    if (tid < NB) {
-      // lane k owns column k of the top block (pv) and of G (g)
-      const int k = tid;
-      T pv[NB], g[NB];
+    if (wave == 0) {
+      // Lanes 0..31 hold the top block E, lanes 32..63 the Gram matrix G: lane k of either half owns
+      // column k of its matrix (x[q] = entry q).  A step needs entry q of column t of E in every lane
+      // of the lower half and entry q of column t of G (= G[t][q], its symmetric twin) in every lane
+      // of the upper half: one broadcast inside each half of the wavefront serves both, and one
+      // instruction stream updates both matrices,
+      //   E[q][k] -= tc_k (E[q][t] s)
+      //   G[q][k] -= tc_k (G[q][t] s) + tc_q u_k,   u_k = s G[t][k] - tc_k s^2 G[t][t]
+      // (the correction <a'_q,a'_k> = <a_q,a_k> - tc_k s<a_t,a_q> - tc_q s<a_t,a_k> + tc_q tc_k s^2<a_t,a_t>).
+      const int k = lane & (NB - 1);
+      const bool upper = lane >= NB;
+      T x[NB];
 #pragma unroll
-      for (int q = 0; q < NB; ++q) {
-        pv[q] = s_piv[q * NB + k];
-        g[q] = s_tot[q * NB + k];
-      }
-      T size_diag = fabsf(s_tot[k * NB + k]);  // size of the terms G[k][k] is made of
+      for (int q = 0; q < NB; ++q) x[q] = upper ? s_tot[q * NB + k] : s_piv[q * NB + k];
+      T size_diag = fabsf(s_tot[k * NB + k]);  // size of the terms G[k][k] is made of (same in both halves)
       T seen = s_seen;
       int done = c;
       bool open = true;
@@ -824,22 +842,45 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       static_for<0, NB>([&](auto step) {
         constexpr int t = decltype(step)::value;
         if (t >= c && t < nbw) {
-          // e_k = <column t, column k> over the explicit rows below pivot t; lane t's value is the
-          // explicit part of column t's squared norm.  Broadcasts go four at a time so that the
-          // scalar results are not needed by the very next instruction.
-          T e = T(0);
-          static_for_by4<t + 1, NB>([&](auto block) {
-            constexpr int q = decltype(block)::value;
-            T col[4];
-#pragma unroll
-            for (int b = 0; b < 4; ++b) col[b] = (q + b < NB) ? lane_value<t>(pv[(q + b) & (NB - 1)]) : T(0);
-#pragma unroll
-            for (int b = 0; b < 4; ++b)
-              if (q + b < NB) e += col[b] * pv[(q + b) & (NB - 1)];
+          // (the lane's column number and half are made opaque per step: otherwise the compiler keeps
+          // the 32 masks `k > t` and the half masks live across the whole panel in scalar registers it
+          // does not have, and reloads each from a spill slot with two cross-lane reads)
+          int kk = k, half = upper ? 1 : 0;
+          keep_behind_wait(kk);
+          keep_behind_wait(half);
+          const bool upper_t = half != 0;
+          // b[q] = entry q of column t, broadcast over the half.  All broadcasts of a step are issued
+          // together and waited for once (the compiler, left to place them, waits for each one where
+          // it is used).
+          T b[NB];
+          static_for<t + 1, NB>([&](auto row) {
+            constexpr int q = decltype(row)::value;
+            b[q] = half_broadcast_issue<t>(x[q]);
           });
-          const T alpha = lane_value<t>(pv[t]);
-          const T hidden2 = lane_value<t>(g[t]);
-          const T x2_explicit = lane_value<t>(e);
+          lds_wait_all();
+          static_for<t + 1, NB>([&](auto row) {
+            constexpr int q = decltype(row)::value;
+            keep_behind_wait(b[q]);
+          });
+          // lower half: e_k = <column t, column k> of E over the rows below pivot t
+          T e = T(0);
+          static_for<t + 1, NB>([&](auto row) {
+            constexpr int q = decltype(row)::value;
+            e += b[q] * x[q];
+          });
+          // Both halves need E[t][k], G[t][k] and e_k: a swap of the halves of two copies of a
+          // register leaves the lower half's value in every lane of one and the upper half's in
+          // every lane of the other.
+          unsigned xt_lower = __float_as_uint(x[t]), xt_upper = xt_lower;
+          lane_swap<true>(xt_lower, xt_upper);
+          unsigned e_lower = __float_as_uint(e), e_upper = e_lower;
+          lane_swap<true>(e_lower, e_upper);
+          const T pvt = __uint_as_float(xt_lower);  // E[t][k]
+          const T gt = __uint_as_float(xt_upper);   // G[t][k]
+          const T ek = __uint_as_float(e_lower);
+          const T alpha = lane_value<t>(pvt);
+          const T hidden2 = lane_value<t>(gt);
+          const T x2_explicit = lane_value<t>(ek);
           const T size_t_ = lane_value<t>(size_diag);
           // (the last column of the matrix has nothing below its pivot: exactly zero, so tau = 0 as in LAPACK)
           const T x2 = (p + t < n - 1) ? x2_explicit + fmaxf(hidden2, T(0)) : T(0);
@@ -847,44 +888,25 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
           open = open && (t == c || (finite && alpha * alpha + x2 >= kQrRoundGuard * size_t_));
           const Reflector h = make_reflector_fast(alpha, x2, kQrNegligible * seen);
           seen = open ? fmaxf(seen, alpha * alpha + x2) : seen;  // (what outlives the round must not see a refused step)
-          const T d = g[t] + e;  // <column t, column k> below pivot t
-          const T tc = (k > t) ? h.tau * (pv[t] + h.scale * d) : T(0);
-          s_tc[t][k] = tc;
+          const T d = gt + ek;  // <column t, column k> below pivot t
+          const T tc = (kk > t) ? h.tau * (pvt + h.scale * d) : T(0);
+          if (!upper_t) s_tc[t][k] = tc;
           s_scal[t][0] = h.scale;  // (every lane writes the same two numbers)
           s_scal[t][1] = h.tau;
-          // G[i][k] -= tc_k s G[t][i] + tc_i s G[t][k] - tc_i tc_k s^2 G[t][t]  =  tc_k u_i + tc_i w_k
-          const T w = h.scale * g[t];
+          const T w = h.scale * gt;
           const T s2gtt = h.scale * h.scale * hidden2;
-          const T u = w - tc * s2gtt;
-          static_for_by4<t + 1, NB>([&](auto block) {
-            constexpr int q = decltype(block)::value;
-            T col[4], ui[4], tci[4];
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-              constexpr int last = NB - 1;
-              col[b] = (q + b < NB) ? lane_value<t>(pv[(q + b) & last]) : T(0);
-            }
-            static_for<0, 4>([&](auto bb) {
-              constexpr int b = decltype(bb)::value;
-              if constexpr (q + b < NB) {
-                ui[b] = lane_value<q + b>(u);
-                tci[b] = lane_value<q + b>(tc);
-              }
-            });
-#pragma unroll
-            for (int b = 0; b < 4; ++b)
-              if (q + b < NB) {
-                // explicit rows: E[q][k] -= tc_k (E[q][t] s), rounded exactly as the rows' owners do it
-                // further down, so that both hold the same numbers (lane t itself has tc = 0)
-                pv[(q + b) & (NB - 1)] -= tc * (col[b] * h.scale);
-                g[(q + b) & (NB - 1)] = (g[(q + b) & (NB - 1)] - tc * ui[b]) - tci[b] * w;
-              }
+          const T u = upper_t ? w - tc * s2gtt : T(0);
+          static_for<t + 1, NB>([&](auto row) {
+            constexpr int q = decltype(row)::value;
+            // lower half: rounded exactly as the rows' owners do it further down, so that both hold
+            // the same numbers (u = 0 there; lane t itself has tc = 0)
+            x[q] = (x[q] - tc * (b[q] * h.scale)) - lane_value<q>(tc) * u;
           });
           size_diag += T(2) * fabsf(tc * w) + fabsf(tc * tc * s2gtt);
           done = open ? t + 1 : done;
         }
       });
-      if (k == 0) {
+      if (lane == 0) {
         s_done = done;
         s_seen = seen;
       }
