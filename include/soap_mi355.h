@@ -59,6 +59,10 @@ const char* soapmi_last_error(void);
  *       factorisation chain side by side, the smaller one on a stream the library owns, forked from
  *       and joined back into the caller's stream with events; with 1 everything is enqueued on the
  *       caller's stream, one chain after the other.  The results are the same bit for bit.
+ *   "qr_carry_update"  0 or 1 (default 1): with 1, the update of the rest of a 256-column block with a
+ *       panel's reflectors rides along in the launch of the next panel (extra workgroups update the
+ *       columns behind that panel, the panel's own workgroups update their 32 columns themselves);
+ *       with 0 it is a launch of its own between two panels.
  *   "persistent_workgroup_budget"  1..256 (default 256): the QR panel kernel and the
  *       tridiagonalisation's column kernel need all workgroups of a launch resident together (one per
  *       256 rows).  The library keeps count of the factorisations that may still be running on a

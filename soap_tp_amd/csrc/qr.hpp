@@ -678,13 +678,211 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+// In-block update of a 32-column panel in one launch: C (rows x nc, ld ldc) <- C - V X with
+// X = T^T (V^T C) obtained as in reflector_w2_solve_kernel from the split-K slices of V^T [V | C].
+// A workgroup owns 256 rows and kPanelApplyCols columns.  Every workgroup of a column group sums
+// the slices and solves for X itself (the same numbers in the same order everywhere: 12 KB per
+// slice, a forward substitution of 32 steps with one lane per column), which costs less than a
+// launch of its own; the product then runs on the matrix cores with the roles of rows and columns
+// swapped, D[column][row] += (-X)^T[column][k] V^T[k][row], so that the lanes of a wavefront walk
+// down a column of C and of V (coalesced) and X comes out of LDS.
+constexpr int kPanelApplyCols = 64;
+
+// (bx, by) = the workgroup's row block and column group; `col_first` = the first column of C that is
+// updated at all (earlier ones belong to someone else), a multiple of 32.
+__device__ __forceinline__ void panel_apply_tile(const float* __restrict__ part, int splits, int64_t slab, int nc,
+                                                 const float* __restrict__ tau, const float* __restrict__ V,
+                                                 int64_t ldv, float* __restrict__ C, int64_t ldc, int rows, int bx,
+                                                 int by, int col_first) {
+  using T = float;
+  constexpr int M = kQrNb, NC = kPanelApplyCols;
+  __shared__ __align__(16) T s_g[M][M];   // s_g[i][l] = (V^T V)[i][l], read for i < l
+  __shared__ T s_w[NC][M + 1];            // s_w[c][i] = (V^T C)[i][c] of this column group
+  __shared__ T s_xn[M][NC];               // s_xn[k][c] = -X[k][c]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col0 = col_first + by * NC;
+  // Rows 64 wave .. 64 wave + 63 of the workgroup: two row tiles by two column tiles of 32 x 32.
+  // The tile of C and the rows of V are requested first; they arrive while X is being made.
+  const int64_t row_base = (int64_t)bx * 256 + wave * 64;
+  const int jr = lane & 31, half = lane >> 5;
+  Mfma<T>::Acc acc[2][2];
+  T vb[2][M / 2];
+  // (loads are unconditional: a row past the end reads the last row and is not stored; a column group
+  // that reaches past the last column takes the slower, tested loads)
+  const bool full_cols = col0 + NC <= nc;
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int64_t r = min(row_base + rt * 32 + jr, (int64_t)rows - 1);
+    const T* vrow = V + r + (int64_t)half * ldv;
+    const T* crow = C + r + (int64_t)(col0 + 4 * half) * ldc;
+    if (full_cols) {
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+        for (int v = 0; v < Mfma<T>::NACC; ++v)
+          acc[rt][ct][v] = crow[(int64_t)(ct * 32 + 8 * (v >> 2) + (v & 3)) * ldc];  // column col0 + ct * 32 + acc_row(v, lane)
+    } else {
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+        for (int v = 0; v < Mfma<T>::NACC; ++v) {
+          const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
+          acc[rt][ct][v] = (c < nc) ? C[r + (int64_t)c * ldc] : T(0);
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < M / 2; ++ks) vb[rt][ks] = vrow[(int64_t)(2 * ks) * ldv];
+  }
+  {
+    // Fixed-order sums over the slices, 16 bytes per load: thread tid takes entries 4 tid .. 4 tid + 3
+    // of G (four rows of one column) and two such quadruples of this column group's part of W, which
+    // is one contiguous run of 64 x 32 words in a slice.
+    const int eg = 4 * tid;
+    int offset[3];
+    bool inside[3];
+    offset[0] = eg;
+    inside[0] = true;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int e = eg + 1024 * q, c = col0 + (e >> 5);
+      inside[1 + q] = c < nc;
+      offset[1 + q] = inside[1 + q] ? (M + col0) * M + e : 0;
+    }
+    float4 sum[3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q) sum[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto add4 = [](float4& acc4, const float4& x) {
+      acc4.x += x.x;
+      acc4.y += x.y;
+      acc4.z += x.z;
+      acc4.w += x.w;
+    };
+    int z = 0;
+    for (; z + 8 <= splits; z += 8) {  // eight slices' loads in flight
+      float4 v[8][3];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int q = 0; q < 3; ++q) v[u][q] = *reinterpret_cast<const float4*>(part + (int64_t)(z + u) * slab + offset[q]);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int q = 0; q < 3; ++q) add4(sum[q], v[u][q]);
+    }
+    for (; z < splits; ++z) {
+      float4 v[3];
+#pragma unroll
+      for (int q = 0; q < 3; ++q) v[q] = *reinterpret_cast<const float4*>(part + (int64_t)z * slab + offset[q]);
+#pragma unroll
+      for (int q = 0; q < 3; ++q) add4(sum[q], v[q]);
+    }
+    {
+      const int row = eg & 31, col = eg >> 5;
+      s_g[row][col] = sum[0].x;
+      s_g[row + 1][col] = sum[0].y;
+      s_g[row + 2][col] = sum[0].z;
+      s_g[row + 3][col] = sum[0].w;
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int e = eg + 1024 * q, row = e & 31, col = e >> 5;
+      const float4 t = inside[1 + q] ? sum[1 + q] : make_float4(0.f, 0.f, 0.f, 0.f);
+      s_w[col][row] = t.x;
+      s_w[col][row + 1] = t.y;
+      s_w[col][row + 2] = t.z;
+      s_w[col][row + 3] = t.w;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // x_i = tau_i (w_i - sum_{l < i} G[l][i] x_l), one lane per column.  G comes out of registers
+    // (lane l holds column l of G; an entry is read across lanes into a scalar): with the entries
+    // in LDS every pair of multiply-adds waited for its own LDS read.
+    T w[M], gcol[M];
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      w[i] = s_w[lane][i];
+      gcol[i] = s_g[i][lane & 31];
+    }
+    static_for<0, M>([&](auto step) {
+      constexpr int i = decltype(step)::value;
+      const T xi = tau[i] * w[i];
+      s_xn[i][lane] = -xi;
+      static_for<i + 1, M>([&](auto col) {
+        constexpr int l = decltype(col)::value;
+        w[l] -= lane_value<l>(gcol[i]) * xi;
+      });
+    });
+  }
+  __syncthreads();
+#pragma unroll
+  for (int ks = 0; ks < M / 2; ++ks) {
+    const int k = 2 * ks + half;
+    T a[2];
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) a[ct] = s_xn[k][ct * 32 + jr];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct) acc[rt][ct] = Mfma<T>::mma(a[ct], vb[rt][ks], acc[rt][ct]);
+  }
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      const int64_t r = row_base + rt * 32 + jr;
+#pragma unroll
+      for (int v = 0; v < Mfma<T>::NACC; ++v) {
+        const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
+        if (r < rows && c < nc) C[r + (int64_t)c * ldc] = acc[rt][ct][v];
+      }
+    }
+}
+
+__global__ __launch_bounds__(256) void panel_apply_kernel(const float* __restrict__ part, int splits, int64_t slab,
+                                                          int nc, const float* __restrict__ tau,
+                                                          const float* __restrict__ V, int64_t ldv,
+                                                          float* __restrict__ C, int64_t ldc, int rows) {
+  panel_apply_tile(part, splits, slab, nc, tau, V, ldv, C, ldc, rows, blockIdx.x, blockIdx.y, 0);
+}
+
+// The panel before this one in the same outer block, when its in-block update rides along in this
+// launch (`slices` null: it does not).  The first `apply_wgs` workgroups of the grid then update
+// the columns behind this panel with the earlier panel's reflectors (panel_apply_tile; they wait for
+// nobody), and the panel's own workgroups first bring their 32 columns up to date themselves, in
+// registers, from the same slices.  Before a panel workgroup reads the columns behind the panel (for
+// its own slice product) it waits until `done_counter` has reached `done_target`, i.e. until every
+// updating workgroup of this launch has finished; the counter only ever grows, so it needs no reset.
+struct PanelCarry {
+  const float* slices;   // the earlier panel's slices of V^T [V | C]
+  int splits;            // number of slices
+  int64_t slab;          // words per slice
+  int nc;                // columns of C behind the earlier panel (the first 32 are this panel)
+  const float* tau;      // the earlier panel's 32 tau
+  const float* v;        // its reflectors, element (row p of this panel, column 0); ld ldv
+  int apply_wgs, apply_row_blocks;
+  unsigned* done_counter;
+  unsigned done_target;
+};
+
 __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ A, int64_t lda, int n, int p, int pe,
                                                             unsigned long long* part, unsigned long long* piv,
                                                             float* __restrict__ tau, unsigned seq_base, int* error,
                                                             int nwg, unsigned spin_limit, float* __restrict__ vout,
                                                             int64_t ldv, int vrow0, float* __restrict__ slices, int nc,
-                                                            int64_t slab) {
+                                                            int64_t slab, PanelCarry carry) {
   using T = float;
+  if (carry.slices != nullptr && (int)blockIdx.x < carry.apply_wgs) {
+    // ---- the earlier panel's update of the columns behind this panel ----
+    const int bx = (int)blockIdx.x % carry.apply_row_blocks, by = (int)blockIdx.x / carry.apply_row_blocks;
+    panel_apply_tile(carry.slices, carry.splits, carry.slab, carry.nc, carry.tau, carry.v, ldv,
+                     A + p + (int64_t)p * lda, lda, n - p, bx, by, kQrNb);
+    // make the columns visible to the whole device, then count this workgroup as done
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(carry.done_counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
   constexpr int NB = kQrNb, GW = kQrGramWords, XS = NB + 1;
   static_assert(GW == 512 + 16, "the exchange below splits the Gram values as 2 x 256 + 16");
   __shared__ T s_x[4][64 * XS];  // a wavefront's rows on their way to the MFMA layout, then its Gram matrix
@@ -698,7 +896,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
   __shared__ int s_done;
   __shared__ int s_fail;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wg = blockIdx.x;
+  const int wg = (int)blockIdx.x - (carry.slices != nullptr ? carry.apply_wgs : 0);
   const int r = p + wg * 256 + tid;
   const int nbw = pe - p;
   const bool live = r < n;
@@ -719,6 +917,118 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     for (int k = 0; k < NB; ++k) {
       const T x = arow[(int64_t)min(k, nbw - 1) * lda];
       a[k] = (live && k < nbw) ? x : T(0);
+    }
+  }
+
+  if (carry.slices != nullptr) {
+    // ---- this panel's columns brought up to date with the earlier panel's reflectors ----
+    // a[c] -= sum_t V[r][t] X[t][c], X = T^T (V^T C) for the first 32 columns of C, from the slices
+    // as in panel_apply_tile: fixed-order sums (16-byte loads), then the forward substitution with
+    // one lane per column.  Every workgroup computes the same X.
+    __shared__ __align__(16) T s_cg[NB][NB];   // s_cg[i][l] = (V^T V)[i][l]
+    __shared__ T s_cw[NB][NB + 1];             // s_cw[c][i] = (V^T C)[i][c]
+    __shared__ __align__(16) T s_cx[NB][NB];   // s_cx[t][c] = -X[t][c]
+    // The product runs on the matrix cores as in panel_apply_tile (operand b = V with lane = row of a
+    // 32-row tile, requested now and used after X is known).
+    const int jr = lane & 31, half = lane >> 5;
+    T vb[2][NB / 2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+      const int rl = min(wg * 256 + wave * 64 + rt * 32 + jr, n - 1 - p);  // row of the tile, relative to row p
+      const T* vp = carry.v + rl + (int64_t)half * ldv;
+#pragma unroll
+      for (int ks = 0; ks < NB / 2; ++ks) vb[rt][ks] = vp[(int64_t)(2 * ks) * ldv];
+    }
+    {
+      const int eg = 4 * tid;  // entries 4 tid .. 4 tid + 3 of G, and of the first 32 columns of W
+      float4 sg = make_float4(0.f, 0.f, 0.f, 0.f), sw = sg;
+      auto add4 = [](float4& acc4, const float4& x) {
+        acc4.x += x.x;
+        acc4.y += x.y;
+        acc4.z += x.z;
+        acc4.w += x.w;
+      };
+      int z = 0;
+      for (; z + 8 <= carry.splits; z += 8) {
+        float4 vg[8], vw[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const float* base = carry.slices + (int64_t)(z + u) * carry.slab;
+          vg[u] = *reinterpret_cast<const float4*>(base + eg);
+          vw[u] = *reinterpret_cast<const float4*>(base + NB * NB + eg);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          add4(sg, vg[u]);
+          add4(sw, vw[u]);
+        }
+      }
+      for (; z < carry.splits; ++z) {
+        const float* base = carry.slices + (int64_t)z * carry.slab;
+        add4(sg, *reinterpret_cast<const float4*>(base + eg));
+        add4(sw, *reinterpret_cast<const float4*>(base + NB * NB + eg));
+      }
+      const int row = eg & (NB - 1), col = eg >> 5;
+      s_cg[row][col] = sg.x;
+      s_cg[row + 1][col] = sg.y;
+      s_cg[row + 2][col] = sg.z;
+      s_cg[row + 3][col] = sg.w;
+      s_cw[col][row] = sw.x;
+      s_cw[col][row + 1] = sw.y;
+      s_cw[col][row + 2] = sw.z;
+      s_cw[col][row + 3] = sw.w;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      T w[NB], gcol[NB];
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        w[i] = s_cw[lane & (NB - 1)][i];
+        gcol[i] = s_cg[i][lane & (NB - 1)];
+      }
+      static_for<0, NB>([&](auto step) {
+        constexpr int i = decltype(step)::value;
+        const T xi = carry.tau[i] * w[i];
+        if (lane < NB) s_cx[i][lane] = -xi;
+        static_for<i + 1, NB>([&](auto col) {
+          constexpr int l = decltype(col)::value;
+          w[l] -= lane_value<l>(gcol[i]) * xi;
+        });
+      });
+    }
+    __syncthreads();
+    {
+      // A thread holds its row in a[0..31]; the accumulator layout of a 32 x 32 tile gives lane l
+      // columns 8 j + i and lane l + 32 columns 8 j + 4 + i (j, i < 4) of row l.  Swapping the upper
+      // half of the registers of one column set with the lower half of the other's turns the two
+      // layouts into each other: before the products, and back after them.
+      Mfma<T>::Acc acc[2];
+#pragma unroll
+      for (int v = 0; v < Mfma<T>::NACC; ++v) {
+        const int c0 = 8 * (v >> 2) + (v & 3);
+        unsigned lo = __float_as_uint(a[c0]), hi = __float_as_uint(a[c0 + 4]);
+        lane_swap<true>(lo, hi);
+        acc[0][v] = __uint_as_float(lo);  // rows 0..31 of the wavefront
+        acc[1][v] = __uint_as_float(hi);  // rows 32..63
+      }
+#pragma unroll
+      for (int ks = 0; ks < NB / 2; ++ks) {
+        const T xk = s_cx[2 * ks + half][jr];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) acc[rt] = Mfma<T>::mma(xk, vb[rt][ks], acc[rt]);
+      }
+#pragma unroll
+      for (int v = 0; v < Mfma<T>::NACC; ++v) {
+        const int c0 = 8 * (v >> 2) + (v & 3);
+        unsigned lo = __float_as_uint(acc[0][v]), hi = __float_as_uint(acc[1][v]);
+        lane_swap<true>(lo, hi);
+        a[c0] = __uint_as_float(lo);
+        a[c0 + 4] = __uint_as_float(hi);
+      }
+    }
+    if (!live) {
+#pragma unroll
+      for (int k = 0; k < NB; ++k) a[k] = T(0);
     }
   }
 
@@ -936,6 +1246,28 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     c = done;
   }
   if (slices == nullptr) return;
+  if (carry.slices != nullptr && carry.apply_wgs > 0) {
+    // the columns behind the panel are being updated by the first workgroups of this launch
+    if (tid == 0) {
+      unsigned polls = 0;
+      bool ok = true;
+      while (__hip_atomic_load(carry.done_counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) - carry.done_target >
+             0x7fffffffu) {  // (counter still behind the target, in wrap-around arithmetic)
+        if (++polls > spin_limit) {
+          ok = false;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      if (!ok) {
+        __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_fail = 1;
+      }
+    }
+    __syncthreads();
+    if (s_fail) return;
+    __threadfence();
+  }
   // ---- this workgroup's slice of V^T [V | C] ------------------------------------------------------
   // C = the nc columns behind the panel (the rest of the outer block), V = the panel's reflectors,
   // both over this workgroup's 256 rows.  The in-block update needs the sums of these slices over
@@ -1357,165 +1689,6 @@ __global__ __launch_bounds__(256) void reflector_w2_solve_kernel(const T* __rest
   if (mine) W2[l + (int64_t)c * ldw2] = x;
 }
 
-// In-block update of a 32-column panel in one launch: C (rows x nc, ld ldc) <- C - V X with
-// X = T^T (V^T C) obtained as in reflector_w2_solve_kernel from the split-K slices of V^T [V | C].
-// A workgroup owns 256 rows and kPanelApplyCols columns.  Every workgroup of a column group sums
-// the slices and solves for X itself (the same numbers in the same order everywhere: 12 KB per
-// slice, a forward substitution of 32 steps with one lane per column), which costs less than a
-// launch of its own; the product then runs on the matrix cores with the roles of rows and columns
-// swapped, D[column][row] += (-X)^T[column][k] V^T[k][row], so that the lanes of a wavefront walk
-// down a column of C and of V (coalesced) and X comes out of LDS.
-constexpr int kPanelApplyCols = 64;
-
-__global__ __launch_bounds__(256) void panel_apply_kernel(const float* __restrict__ part, int splits, int64_t slab,
-                                                          int nc, const float* __restrict__ tau,
-                                                          const float* __restrict__ V, int64_t ldv,
-                                                          float* __restrict__ C, int64_t ldc, int rows) {
-  using T = float;
-  constexpr int M = kQrNb, NC = kPanelApplyCols;
-  __shared__ __align__(16) T s_g[M][M];   // s_g[i][l] = (V^T V)[i][l], read for i < l
-  __shared__ T s_w[NC][M + 1];            // s_w[c][i] = (V^T C)[i][c] of this column group
-  __shared__ T s_xn[M][NC];               // s_xn[k][c] = -X[k][c]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int col0 = blockIdx.y * NC;
-  // Rows 64 wave .. 64 wave + 63 of the workgroup: two row tiles by two column tiles of 32 x 32.
-  // The tile of C and the rows of V are requested first; they arrive while X is being made.
-  const int64_t row_base = (int64_t)blockIdx.x * 256 + wave * 64;
-  const int jr = lane & 31, half = lane >> 5;
-  Mfma<T>::Acc acc[2][2];
-  T vb[2][M / 2];
-  // (loads are unconditional: a row past the end reads the last row and is not stored; a column group
-  // that reaches past the last column takes the slower, tested loads)
-  const bool full_cols = col0 + NC <= nc;
-#pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
-    const int64_t r = min(row_base + rt * 32 + jr, (int64_t)rows - 1);
-    const T* vrow = V + r + (int64_t)half * ldv;
-    const T* crow = C + r + (int64_t)(col0 + 4 * half) * ldc;
-    if (full_cols) {
-#pragma unroll
-      for (int ct = 0; ct < 2; ++ct)
-#pragma unroll
-        for (int v = 0; v < Mfma<T>::NACC; ++v)
-          acc[rt][ct][v] = crow[(int64_t)(ct * 32 + 8 * (v >> 2) + (v & 3)) * ldc];  // column col0 + ct * 32 + acc_row(v, lane)
-    } else {
-#pragma unroll
-      for (int ct = 0; ct < 2; ++ct)
-#pragma unroll
-        for (int v = 0; v < Mfma<T>::NACC; ++v) {
-          const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
-          acc[rt][ct][v] = (c < nc) ? C[r + (int64_t)c * ldc] : T(0);
-        }
-    }
-#pragma unroll
-    for (int ks = 0; ks < M / 2; ++ks) vb[rt][ks] = vrow[(int64_t)(2 * ks) * ldv];
-  }
-  {
-    // Fixed-order sums over the slices, 16 bytes per load: thread tid takes entries 4 tid .. 4 tid + 3
-    // of G (four rows of one column) and two such quadruples of this column group's part of W, which
-    // is one contiguous run of 64 x 32 words in a slice.
-    const int eg = 4 * tid;
-    int offset[3];
-    bool inside[3];
-    offset[0] = eg;
-    inside[0] = true;
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const int e = eg + 1024 * q, c = col0 + (e >> 5);
-      inside[1 + q] = c < nc;
-      offset[1 + q] = inside[1 + q] ? (M + col0) * M + e : 0;
-    }
-    float4 sum[3];
-#pragma unroll
-    for (int q = 0; q < 3; ++q) sum[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-    auto add4 = [](float4& acc4, const float4& x) {
-      acc4.x += x.x;
-      acc4.y += x.y;
-      acc4.z += x.z;
-      acc4.w += x.w;
-    };
-    int z = 0;
-    for (; z + 8 <= splits; z += 8) {  // eight slices' loads in flight
-      float4 v[8][3];
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-#pragma unroll
-        for (int q = 0; q < 3; ++q) v[u][q] = *reinterpret_cast<const float4*>(part + (int64_t)(z + u) * slab + offset[q]);
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-#pragma unroll
-        for (int q = 0; q < 3; ++q) add4(sum[q], v[u][q]);
-    }
-    for (; z < splits; ++z) {
-      float4 v[3];
-#pragma unroll
-      for (int q = 0; q < 3; ++q) v[q] = *reinterpret_cast<const float4*>(part + (int64_t)z * slab + offset[q]);
-#pragma unroll
-      for (int q = 0; q < 3; ++q) add4(sum[q], v[q]);
-    }
-    {
-      const int row = eg & 31, col = eg >> 5;
-      s_g[row][col] = sum[0].x;
-      s_g[row + 1][col] = sum[0].y;
-      s_g[row + 2][col] = sum[0].z;
-      s_g[row + 3][col] = sum[0].w;
-    }
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const int e = eg + 1024 * q, row = e & 31, col = e >> 5;
-      const float4 t = inside[1 + q] ? sum[1 + q] : make_float4(0.f, 0.f, 0.f, 0.f);
-      s_w[col][row] = t.x;
-      s_w[col][row + 1] = t.y;
-      s_w[col][row + 2] = t.z;
-      s_w[col][row + 3] = t.w;
-    }
-  }
-  __syncthreads();
-  if (wave == 0) {
-    // x_i = tau_i (w_i - sum_{l < i} G[l][i] x_l), one lane per column.  G comes out of registers
-    // (lane l holds column l of G; an entry is read across lanes into a scalar): with the entries
-    // in LDS every pair of multiply-adds waited for its own LDS read.
-    T w[M], gcol[M];
-#pragma unroll
-    for (int i = 0; i < M; ++i) {
-      w[i] = s_w[lane][i];
-      gcol[i] = s_g[i][lane & 31];
-    }
-    static_for<0, M>([&](auto step) {
-      constexpr int i = decltype(step)::value;
-      const T xi = tau[i] * w[i];
-      s_xn[i][lane] = -xi;
-      static_for<i + 1, M>([&](auto col) {
-        constexpr int l = decltype(col)::value;
-        w[l] -= lane_value<l>(gcol[i]) * xi;
-      });
-    });
-  }
-  __syncthreads();
-#pragma unroll
-  for (int ks = 0; ks < M / 2; ++ks) {
-    const int k = 2 * ks + half;
-    T a[2];
-#pragma unroll
-    for (int ct = 0; ct < 2; ++ct) a[ct] = s_xn[k][ct * 32 + jr];
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < 2; ++ct) acc[rt][ct] = Mfma<T>::mma(a[ct], vb[rt][ks], acc[rt][ct]);
-  }
-#pragma unroll
-  for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-    for (int ct = 0; ct < 2; ++ct) {
-      const int64_t r = row_base + rt * 32 + jr;
-#pragma unroll
-      for (int v = 0; v < Mfma<T>::NACC; ++v) {
-        const int c = col0 + ct * 32 + Mfma<T>::acc_row(v, lane);
-        if (r < rows && c < nc) C[r + (int64_t)c * ldc] = acc[rt][ct][v];
-      }
-    }
-}
-
 template <typename T>
 static inline int gram_of_v(hipStream_t s, const BlockReflectorWs<T>& ws, int rows, int nbw, int64_t ldv) {
   using Skinny = typename SkinnyTile<T>::type;
@@ -1591,7 +1764,7 @@ struct QrWorkspace {
   T* piv;     // 2 x NB
   unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x kQrMailWords   mailboxes of the persistent panel kernels
   unsigned long long* mail_piv;   // 2 x kQrMailPivotWords
-  unsigned* sync;  // [1] error flag of the persistent panel kernel
+  unsigned* sync;  // [1] error flag of the persistent panel kernel, [2] count of finished updating workgroups
 };
 
 template <typename T, class WS>
@@ -1625,13 +1798,14 @@ template <typename T>
 static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
                                        const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
                                        unsigned spin_limit = kQrSpinLimit, int columns_per_round = kQrRoundMax,
-                                       int* report = nullptr) {
+                                       int* report = nullptr, bool carry_updates = true) {
   const int NB = kQrNb, OB = kBrMax;
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
   int rc;
   static_assert(std::is_same<T, float>::value, "the persistent panel kernel packs float values into its mailboxes");
   unsigned seq_base = 0;
+  unsigned carried_total = 0;  // updating workgroups issued so far (what ws.sync[2] counts up to)
   hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
   {
     // sequence number 0 = "nothing yet"; mail_piv follows mail_part in the workspace, one clear covers both
@@ -1647,6 +1821,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     hipLaunchKernelGGL((fill_zero_kernel<T>), dim3(OB * OB / 256), dim3(256), 0, s, Tm, OB * OB);
     int inner_done = 0;
     bool v_written = true;  // the panel kernels leave the block's reflectors in ws.br.v
+    int pending_p = -1, pending_nwg = 0, pending_buffer = 0;  // a panel whose in-block update has not been issued
     for (int p = P; p < PE; p += NB) {
       const int pe = std::min(PE, p + NB), nbw = pe - p;
       const int rows = n - p;
@@ -1658,13 +1833,54 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
       inner.v = ws.br.v + (p - P) + (int64_t)(p - P) * ldv;
       bool slices_by_panel = false;
       if (nwg <= persistent_max_wg && columns_per_round == kQrWholePanel) {
-        // (a full panel with columns of the outer block behind it also leaves its slices of V^T [V | C])
+        // (a full panel with columns of the outer block behind it also leaves its slices of V^T [V | C];
+        // two slice buffers alternate, since a launch may read the earlier panel's while writing its own)
         slices_by_panel = pe < PE && nbw == NB;
-        hipLaunchKernelGGL(qr_panel_gram_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part, ws.mail_piv,
-                           ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
-                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, slices_by_panel ? ws.br.splitk : nullptr, PE - pe,
-                           (int64_t)NB * (PE - p));
+        T* slice_buffer[2] = {ws.br.splitk, ws.br.splitk + (size_t)kBrSplits * kBrMax * ldv / 2};
+        PanelCarry carry{};
+        if (pending_p >= 0 && nbw == NB) {
+          // the earlier panel's in-block update rides along in this launch
+          const int groups = (int)ceil_div64(PE - pe, kPanelApplyCols);
+          carry.slices = slice_buffer[pending_buffer];
+          carry.splits = pending_nwg;
+          carry.slab = (int64_t)NB * (PE - pending_p);
+          carry.nc = PE - p;
+          carry.tau = ws.tau + pending_p;
+          carry.v = ws.br.v + (p - P) + (int64_t)(pending_p - P) * ldv;
+          carry.apply_row_blocks = nwg;
+          carry.apply_wgs = nwg * groups;
+          carry.done_counter = ws.sync + 2;
+          carried_total += (unsigned)carry.apply_wgs;
+          carry.done_target = carried_total;
+          pending_p = -1;
+        } else if (pending_p >= 0) {
+          // (a last, narrower panel: the earlier panel's update as a launch of its own)
+          hipLaunchKernelGGL(panel_apply_kernel,
+                             dim3((unsigned)ceil_div64(n - pending_p, 256), (unsigned)ceil_div64(PE - p, kPanelApplyCols)),
+                             dim3(256), 0, s, slice_buffer[pending_buffer], pending_nwg, (int64_t)NB * (PE - pending_p),
+                             PE - p, ws.tau + pending_p, ws.br.v + (pending_p - P) + (int64_t)(pending_p - P) * ldv, ldv,
+                             A + pending_p + (int64_t)p * lda, lda, n - pending_p);
+          SOAPMI_LAUNCH_CHECK();
+          pending_p = -1;
+        }
+        const int out_buffer = pending_buffer ^ 1;
+        hipLaunchKernelGGL(qr_panel_gram_kernel, dim3(nwg + carry.apply_wgs), dim3(256), 0, s, A, lda, n, p, pe,
+                           ws.mail_part, ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
+                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, slices_by_panel ? slice_buffer[out_buffer] : nullptr,
+                           PE - pe, (int64_t)NB * (PE - p), carry);
         seq_base += (unsigned)nbw;
+        if (slices_by_panel) {
+          pending_buffer = out_buffer;
+          if (carry_updates) {
+            pending_p = p;
+            pending_nwg = nwg;
+          } else {
+            hipLaunchKernelGGL(panel_apply_kernel,
+                               dim3((unsigned)nwg, (unsigned)ceil_div64(PE - pe, kPanelApplyCols)), dim3(256), 0, s,
+                               slice_buffer[out_buffer], nwg, (int64_t)NB * (PE - p), PE - pe, ws.tau + p, inner.v, ldv,
+                               A + p + (int64_t)pe * lda, lda, rows);
+          }
+        }
       } else if (nwg <= persistent_max_wg) {
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
                            ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
@@ -1679,20 +1895,20 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
         v_written = false;
       }
       SOAPMI_LAUNCH_CHECK();
-      if (pe < PE && v_written) {
+      if (slices_by_panel) {
+        // (the in-block update is on its way or rides along with the next panel)
+      } else if (pe < PE && v_written) {
         // The panel's reflectors act on the rest of the outer block only.  One product gives the
         // slices of V^T [V | C] (the panel's own columns of A hold V in clean form); the middle
         // factor T^T is applied as a triangular solve with V^T V, so no T is needed here: the
         // diagonal blocks of the outer factor are all built after the block's last panel.
         using Skinny = typename SkinnyTile<T>::type;
         const int ncols = PE - p, nc = PE - pe;
-        int slices = nwg;
-        if (!slices_by_panel) {
-          rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, ncols, rows, inner.v, ldv, A + p + (int64_t)p * lda, lda,
-                                           split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
-                                           ws.br.splitk, &slices);
-          if (rc) return rc;
-        }
+        int slices = 1;
+        rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, ncols, rows, inner.v, ldv, A + p + (int64_t)p * lda, lda,
+                                         split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
+                                         ws.br.splitk, &slices);
+        if (rc) return rc;
         if (nbw == NB) {
           hipLaunchKernelGGL(panel_apply_kernel, dim3((unsigned)ceil_div64(rows, 256), (unsigned)ceil_div64(nc, kPanelApplyCols)),
                              dim3(256), 0, s, ws.br.splitk, slices, (int64_t)nbw * ncols, nc, ws.tau + p, inner.v, ldv,
