@@ -205,6 +205,28 @@ def test_qr_launch_per_column_panel_path(size, device):
         _native.call("soapmi_set_option", b"qr_persistent_max_workgroups", 129)
 
 
+@pytest.mark.parametrize("size", [96, 300, 545, 1000, 1312])
+def test_qr_update_riding_along_with_the_next_panel(size, device):
+    """A panel's update of the rest of its 256-column block either rides along in the next panel's
+    launch (the default) or is a launch of its own: the same sums in the same order, so the same bits.
+    Sizes with a last panel narrower than 32 columns take the separate launch for that panel."""
+    from soap_tp_amd import _native
+    matrix = make_matrix(size, size, seed=SEED + 7 * size)
+    results = []
+    try:
+        for carried in (0, 1):
+            _native.call("soapmi_set_option", b"qr_carry_update", carried)
+            factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+            ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
+            results.append(factor.cpu())
+    finally:
+        _native.call("soapmi_set_option", b"qr_carry_update", 1)
+    assert relative_l2(results[1], oracle.householder_qr(matrix)) <= 5e-5
+    assert torch.equal(results[0], results[1])
+    with pytest.raises(ValueError):
+        _native.call("soapmi_set_option", b"qr_carry_update", 2)
+
+
 @pytest.mark.parametrize("size", [289, 545, 1000])
 def test_qr_block_reflector_widths(size, device):
     """Sizes whose last 256-column block reflector has a width that is no multiple of 32, 64 or 128:
