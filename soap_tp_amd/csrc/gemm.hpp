@@ -118,9 +118,13 @@ struct EpiAdam {
 // every K-slab and the groups' accumulators are added through LDS before the epilogue.  For tiles
 // so small that a wavefront holds a single accumulator block, this puts two wavefronts on every
 // SIMD, so that one's LDS waits hide behind the other's matrix instructions.
-template <typename T, int BM_, int BN_, int BK_, int WM_, int WN_, int KS_ = 1>
+// PF_ > 1 (fast path only): that many K-slabs are on their way from memory at any time, held in
+// registers until their turn to be stored to LDS.  A tile that runs one workgroup per compute unit
+// has nobody to hide a slab's trip from memory behind; with one slab in flight its loop waits for
+// memory once per slab.
+template <typename T, int BM_, int BN_, int BK_, int WM_, int WN_, int KS_ = 1, int PF_ = 1>
 struct GemmTile {
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, KS = KS_;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, KS = KS_, PF = PF_;
   static constexpr int NT = 64 * WM * WN * KS;
   static constexpr int MI = Mfma<T>::MI, KI = Mfma<T>::KI;
   static constexpr int TM = BM / WM / MI, TN = BN / WN / MI;
@@ -321,12 +325,22 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
   FastLoader<T, BM, BK, NT, Cfg::NVA, AXC> fa;
   FastLoader<T, BN, BK, NT, Cfg::NVB, BXC> fb;
 
+  constexpr int PF = FAST ? Cfg::PF : 1;
+  T pa[PF][Cfg::NVA][VW], pb[PF][Cfg::NVB][VW];  // slabs in flight beyond the next one (PF > 1)
   if (nk > 0) {
     if (FAST) {
       fa.init(p.A, p.lda, m0, kbeg, tid);
       fb.init(p.B, p.ldb, n0, kbeg, tid);
       fa.load(ra);
       fb.load(rb);
+      if constexpr (PF > 1) {
+#pragma unroll
+        for (int sl = 1; sl <= PF; ++sl)
+          if (sl < nk) {
+            fa.load(pa[sl % PF]);
+            fb.load(pb[sl % PF]);
+          }
+      }
     } else {
       load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, kbeg, kend, a_xc, p.vecA, tid);
       load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, kbeg, kend, b_xc, p.vecB, tid, p.ksel_b);
@@ -337,18 +351,7 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
   __syncthreads();
 
   const int krow = lane / MI, idx = lane % MI;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) {
-      if (FAST) {
-        fa.load(ra);
-        fb.load(rb);
-      } else {
-        const int k0 = kbeg + (kt + 1) * BK;
-        load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, k0, kend, a_xc, p.vecA, tid);
-        load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, k0, kend, b_xc, p.vecB, tid, p.ksel_b);
-      }
-    }
+  auto multiply_slab = [&](int buf) {
     const T* as = As[buf];
     const T* bs = Bs[buf];
 #pragma unroll
@@ -364,11 +367,50 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(fn[j], fm[i], acc[i][j]);
     }
-    if (kt + 1 < nk) {
-      store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[buf ^ 1], ra, a_xc, tid);
-      store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[buf ^ 1], rb, b_xc, tid);
+  };
+  if constexpr (PF > 1) {
+    // Slab kt + 1 waits in register slot (kt + 1) % PF; once it has been stored to LDS the slot takes
+    // the load of slab kt + 1 + PF.  The loop is unrolled by PF so that slots are compile-time indices.
+    for (int kt0 = 0; kt0 < nk; kt0 += PF) {
+#pragma unroll
+      for (int u = 0; u < PF; ++u) {
+        const int kt = kt0 + u;
+        if (kt < nk) {
+          const int buf = kt & 1;
+          multiply_slab(buf);
+          const int slot = (u + 1) % PF;
+          if (kt + 1 < nk) {
+            store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[buf ^ 1], pa[slot], a_xc, tid);
+            store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[buf ^ 1], pb[slot], b_xc, tid);
+          }
+          if (kt + 1 + PF < nk) {
+            fa.load(pa[slot]);
+            fb.load(pb[slot]);
+          }
+          __syncthreads();
+        }
+      }
     }
-    __syncthreads();
+  } else {
+    for (int kt = 0; kt < nk; ++kt) {
+      const int buf = kt & 1;
+      if (kt + 1 < nk) {
+        if (FAST) {
+          fa.load(ra);
+          fb.load(rb);
+        } else {
+          const int k0 = kbeg + (kt + 1) * BK;
+          load_slab<T, BM, BK, NT, Cfg::NVA>(ra, p.A, p.lda, m0, p.M, k0, kend, a_xc, p.vecA, tid);
+          load_slab<T, BN, BK, NT, Cfg::NVB>(rb, p.B, p.ldb, n0, p.N, k0, kend, b_xc, p.vecB, tid, p.ksel_b);
+        }
+      }
+      multiply_slab(buf);
+      if (kt + 1 < nk) {
+        store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[buf ^ 1], ra, a_xc, tid);
+        store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[buf ^ 1], rb, b_xc, tid);
+      }
+      __syncthreads();
+    }
   }
 
   if constexpr (KS > 1) {
@@ -509,7 +551,7 @@ struct SmallTile {
 // wavefronts split each (32 deep) K-slab between them.
 template <>
 struct SmallTile<float> {
-  using type = GemmTile<float, 64, 64, 32, 2, 2, 2>;
+  using type = GemmTile<float, 64, 64, 32, 2, 2, 2, 2>;
 };
 
 // True if an M x N output has so few default tiles that the 256 CUs are badly filled: at most half
