@@ -906,7 +906,13 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     s_seen = T(0);
   }
   if (wg == 0) {
-    for (int t = tid; t < (p - vrow0) * nbw; t += 256) vout[t % (p - vrow0) + (int64_t)(t / (p - vrow0)) * ldv] = T(0);
+    // rows of the outer block above this panel: zero in the reflector buffer and in A (the entries of
+    // R there have no reader), so that the block's columns of A hold V in clean form as well
+    for (int t = tid; t < (p - vrow0) * nbw; t += 256) {
+      const int row = t % (p - vrow0), col = t / (p - vrow0);
+      vout[row + (int64_t)col * ldv] = T(0);
+      A[(vrow0 + row) + (int64_t)(p + col) * lda] = T(0);
+    }
   }
 
   T a[NB];  // a[k] = A[r, p + k]
@@ -1740,6 +1746,28 @@ static inline int apply_block_reflector(hipStream_t s, const BlockReflectorWs<T>
   return gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), ws.v, ldv, ws.w2, kBrMax, T(1), C, ldc);
 }
 
+// The same for the trailing columns of a factorisation whose panel kernels left V in clean form in
+// the block's own columns of A as well: those columns and the trailing ones are neighbours in A, so
+// one product gives V^T [V | C], i.e. the Gram matrix the T factor is built from and W.
+// `block` = element (first row, first column) of the outer block in A; T (ld kBrMax) is assembled here.
+template <typename T>
+static inline int factor_and_apply_block_reflector(hipStream_t s, const BlockReflectorWs<T>& ws, T* Tm, int rows,
+                                                   int nbw, int nc, int64_t ldv, T* block, int64_t lda, const T* tau,
+                                                   int first_block) {
+  using Wide = typename DefaultTile<T>::type;
+  const int64_t tiles = ceil_div64(nbw + nc, Wide::BN) * ceil_div64(nbw, Wide::BM);
+  const int splits = split_count(tiles, rows, nbw, nbw + nc, ldv);
+  int rc = gemm<T>(s, 1, 0, nbw, nbw + nc, rows, T(1), ws.v, ldv, block, lda, T(0), ws.w, kBrMax, splits, ws.splitk);
+  if (rc) return rc;
+  BlockReflectorWs<T> gram_in_w = ws;
+  gram_in_w.gram = ws.w;
+  rc = assemble_t_factor<T>(s, gram_in_w, nbw, tau, Tm, first_block);
+  if (rc || nc <= 0) return rc;
+  rc = gemm<T>(s, 1, 0, nbw, nc, nbw, T(1), Tm, kBrMax, ws.w + (int64_t)nbw * kBrMax, kBrMax, T(0), ws.w2, kBrMax);
+  if (rc) return rc;
+  return gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), ws.v, ldv, ws.w2, kBrMax, T(1), block + (int64_t)nbw * lda, lda);
+}
+
 template <typename T>
 static inline void launch_extract_v(hipStream_t s, const T* A, int64_t lda, int rows, int row0, int col0, int nbw,
                                     T* V, int64_t ldv, int shift = 0) {
@@ -1822,6 +1850,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     int inner_done = 0;
     bool v_written = true;  // the panel kernels leave the block's reflectors in ws.br.v
     int pending_p = -1, pending_nwg = 0, pending_buffer = 0;  // a panel whose in-block update has not been issued
+    bool clean_in_a = true;  // every panel so far left V in clean form in A too (the whole-panel kernel does)
     for (int p = P; p < PE; p += NB) {
       const int pe = std::min(PE, p + NB), nbw = pe - p;
       const int rows = n - p;
@@ -1882,6 +1911,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
           }
         }
       } else if (nwg <= persistent_max_wg) {
+        clean_in_a = false;
         hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
                            ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
                            ws.br.v + (int64_t)(p - P) * ldv, ldv, P, columns_per_round);
@@ -1893,6 +1923,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
                              piv[in], part[out], piv[out], ws.tau, nwg);
         }
         v_written = false;
+        clean_in_a = false;
       }
       SOAPMI_LAUNCH_CHECK();
       if (slices_by_panel) {
@@ -1939,13 +1970,20 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     }
     const int rows = n - P;
     if (!v_written) launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
-    rc = gram_of_v<T>(s, ws.br, rows, obw, ldv);
-    if (rc) return rc;
-    rc = assemble_t_factor<T>(s, ws.br, obw, ws.tau + P, Tm, inner_done);
-    if (rc) return rc;
-    // trailing columns: C <- H^T C = C - V T^T V^T C
-    rc = apply_block_reflector<T>(s, ws.br, Tm, true, rows, obw, n - PE, ldv, A + P + (int64_t)PE * lda, lda);
-    if (rc) return rc;
+    if (clean_in_a && obw > kQrNb) {
+      // T and the trailing columns, C <- H^T C = C - V T^T V^T C, from one product V^T [V | C]
+      rc = factor_and_apply_block_reflector<T>(s, ws.br, Tm, rows, obw, n - PE, ldv, A + P + (int64_t)P * lda, lda,
+                                               ws.tau + P, inner_done);
+      if (rc) return rc;
+    } else {
+      rc = gram_of_v<T>(s, ws.br, rows, obw, ldv);
+      if (rc) return rc;
+      rc = assemble_t_factor<T>(s, ws.br, obw, ws.tau + P, Tm, inner_done);
+      if (rc) return rc;
+      // trailing columns: C <- H^T C = C - V T^T V^T C
+      rc = apply_block_reflector<T>(s, ws.br, Tm, true, rows, obw, n - PE, ldv, A + P + (int64_t)PE * lda, lda);
+      if (rc) return rc;
+    }
   }
   // ---- explicit Q, outer blocks in reverse ----
   for (int bi = blocks - 1; bi >= 0; --bi) {
