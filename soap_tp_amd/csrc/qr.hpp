@@ -17,6 +17,7 @@
 // compact-WY block reflectors on the MFMA GEMM.
 #pragma once
 #include <type_traits>
+#include <vector>
 
 #include "common.hpp"
 #include "gemm.hpp"
@@ -1834,6 +1835,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
   static_assert(std::is_same<T, float>::value, "the persistent panel kernel packs float values into its mailboxes");
   unsigned seq_base = 0;
   unsigned carried_total = 0;  // updating workgroups issued so far (what ws.sync[2] counts up to)
+  std::vector<char> block_clean((size_t)blocks, 0);  // outer blocks whose columns of A hold V in clean form
   hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
   {
     // sequence number 0 = "nothing yet"; mail_piv follows mail_part in the workspace, one clear covers both
@@ -1970,6 +1972,7 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     }
     const int rows = n - P;
     if (!v_written) launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
+    block_clean[bi] = clean_in_a ? 1 : 0;
     if (clean_in_a && obw > kQrNb) {
       // T and the trailing columns, C <- H^T C = C - V T^T V^T C, from one product V^T [V | C]
       rc = factor_and_apply_block_reflector<T>(s, ws.br, Tm, rows, obw, n - PE, ldv, A + P + (int64_t)P * lda, lda,
@@ -1990,15 +1993,23 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     const int P = bi * OB, PE = std::min(n, P + OB), obw = PE - P;
     const int rows = n - P;
     T* Tm = ws.t_all + (size_t)bi * OB * OB;
-    launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
-    SOAPMI_LAUNCH_CHECK();
+    // V of the block: its columns of A where the panel kernels left them in clean form, else extracted
+    BlockReflectorWs<T> bws = ws.br;
+    int64_t ldvb = ldv;
+    if (block_clean[bi] && lda == ldv) {  // (the split-K buffer is sized by the reflector buffer's leading dimension)
+      bws.v = A + P + (int64_t)P * lda;
+      ldvb = lda;
+    } else {
+      launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
+      SOAPMI_LAUNCH_CHECK();
+    }
     // columns to the right already hold Q of the later blocks: C <- (I - V T V^T) C
-    rc = apply_block_reflector<T>(s, ws.br, Tm, false, rows, obw, n - PE, ldv, Qout + P + (int64_t)PE * ldq, ldq);
+    rc = apply_block_reflector<T>(s, bws, Tm, false, rows, obw, n - PE, ldvb, Qout + P + (int64_t)PE * ldq, ldq);
     if (rc) return rc;
     // own columns: [I;0] - V (T V1^T)
-    rc = gemm<T>(s, 0, 1, obw, obw, obw, T(1), Tm, OB, ws.br.v, ldv, T(0), ws.br.mx, OB);
+    rc = gemm<T>(s, 0, 1, obw, obw, obw, T(1), Tm, OB, bws.v, ldvb, T(0), ws.br.mx, OB);
     if (rc) return rc;
-    rc = gemm<T>(s, 0, 0, rows, obw, obw, T(-1), ws.br.v, ldv, ws.br.mx, OB, T(0), Qout + P + (int64_t)P * ldq, ldq);
+    rc = gemm<T>(s, 0, 0, rows, obw, obw, T(-1), bws.v, ldvb, ws.br.mx, OB, T(0), Qout + P + (int64_t)P * ldq, ldq);
     if (rc) return rc;
     hipLaunchKernelGGL((orgqr_panel_fix_kernel<T>), dim3((unsigned)ceil_div64(PE, 256)), dim3(256), 0, s, Qout, ldq, P,
                        obw);

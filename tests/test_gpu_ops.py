@@ -227,6 +227,26 @@ def test_qr_update_riding_along_with_the_next_panel(size, device):
         _native.call("soapmi_set_option", b"qr_carry_update", 2)
 
 
+@pytest.mark.parametrize("size", [200, 600])
+def test_qr_with_padded_leading_dimensions(size, device):
+    """soapmi_qr_f32 called directly with leading dimensions larger than n, for the matrix and for Q:
+    the factorisation then cannot use the matrix's own columns as the reflector block of the Q formation."""
+    from soap_tp_amd import _native
+    matrix = make_matrix(size, size, seed=SEED + 3 * size)
+    lda, ldq = size + 24, size + 8
+    a_store = torch.full((size, lda), float("nan"), device=device)
+    q_store = torch.full((size, ldq), float("nan"), device=device)
+    a_store[:, :size] = matrix.T.to(device)  # column j of the matrix in row j of the store: column-major with ld = lda
+    need = _native.library().soapmi_qr_workspace_bytes(size)
+    work = torch.empty(need, dtype=torch.uint8, device=device)
+    _native.call("soapmi_qr_f32", a_store.data_ptr(), q_store.data_ptr(), size, lda, ldq, work.data_ptr(), need,
+                 torch.cuda.current_stream().cuda_stream)
+    factor = q_store[:, :size].T.cpu()
+    assert bool(torch.isnan(q_store[:, size:]).all())  # the padding is not written
+    assert relative_l2(factor, oracle.householder_qr(matrix)) <= 5e-5
+    torch.testing.assert_close(factor.T @ factor, torch.eye(size), rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("size", [289, 545, 1000])
 def test_qr_block_reflector_widths(size, device):
     """Sizes whose last 256-column block reflector has a width that is no multiple of 32, 64 or 128:
