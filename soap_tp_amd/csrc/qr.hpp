@@ -1844,11 +1844,12 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3((words + 255) / 256), dim3(256), 0, s,
                        reinterpret_cast<unsigned*>(ws.mail_part), words);
   }
+  // (the T factors of all outer blocks start from zero: one fill instead of one per block)
+  hipLaunchKernelGGL((fill_zero_kernel<T>), dim3(blocks * (OB * OB / 256)), dim3(256), 0, s, ws.t_all, blocks * OB * OB);
   // ---- factorisation ----
   for (int bi = 0; bi < blocks; ++bi) {
     const int P = bi * OB, PE = std::min(n, P + OB), obw = PE - P;
     T* Tm = ws.t_all + (size_t)bi * OB * OB;
-    hipLaunchKernelGGL((fill_zero_kernel<T>), dim3(OB * OB / 256), dim3(256), 0, s, Tm, OB * OB);
     int inner_done = 0;
     bool v_written = true;  // the panel kernels leave the block's reflectors in ws.br.v
     int pending_p = -1, pending_nwg = 0, pending_buffer = 0;  // a panel whose in-block update has not been issued
