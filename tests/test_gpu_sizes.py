@@ -366,3 +366,30 @@ def test_two_stage_eigensolver_at_4096(device):
     finally:
         _native.call("soapmi_set_option", b"eigh_algorithm", 1)
     assert (spectra[0] - spectra[1]).abs().max().item() <= 1e-6 * spectra[0].abs().max().item()
+
+
+def test_qr_with_more_workgroups_in_a_launch_than_compute_units(device):
+    """n = 16640: a panel launch holds 65 panel workgroups and up to 195 workgroups that update the columns
+    behind the panel for the previous one, more than the chip's 256 compute units hold at once.  The
+    updating workgroups come first in the launch and wait for nobody, so the panel's own workgroups are
+    all placed once those have finished.  Checked by properties (a CPU factorisation of this size takes
+    minutes): orthogonality on a sample of columns, ``Q^T A`` upper triangular and the backward error of
+    the leading columns."""
+    size = 16640
+    generator = torch.Generator(device=device).manual_seed(SEED + size)
+    matrix = torch.randn(size, size, device=device, generator=generator).T  # column-major
+    work = matrix.clone()
+    factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+    ops.qr_2d_block_cyclic_(work, factor, size, BLOCK, GRID)
+    torch.cuda.synchronize()
+    assert not soap_tp_amd._native.device_error_flag()
+    sample = torch.cat([torch.arange(0, 256), torch.arange(size // 2, size // 2 + 256),
+                        torch.arange(size - 256, size)]).to(device)
+    q_sample = factor[:, sample].double()
+    identity = torch.eye(sample.numel(), dtype=torch.float64, device=device)
+    assert (q_sample.T @ q_sample - identity).abs().max().item() <= 1e-5
+    lead = 512
+    r_lead = factor[:, :lead].double().T @ matrix[:, :lead].double()
+    assert torch.tril(r_lead, -1).abs().max().item() <= 1e-5 * r_lead.abs().max().item()
+    residual = factor[:, :lead].double() @ torch.triu(r_lead) - matrix[:, :lead].double()
+    assert residual.norm().item() <= 1e-5 * matrix[:, :lead].double().norm().item()
