@@ -199,6 +199,27 @@ def test_step_and_bases_at_benchmark_sizes(shape, rank, implementation, device, 
         assert identity_error.abs().max().item() <= 1e-4
 
 
+SWEEP = [(size, implementation) for size in (16, 32, 64, 128, 256, 512, 2048) for implementation in ("elpa", "eigh")]
+
+
+@pytest.mark.parametrize("size,implementation", SWEEP + [(8192, "elpa"), (8192, "eigh")])
+def test_square_sizes_of_the_reference_accuracy_sweep(size, implementation, device, monkeypatch):
+    """The square sizes of the reference's accuracy sweep that no other test runs
+    (scripts/slurm/frontier/soap_accuracy.slurm:62-68: 8 ... 8192, both variants; 8, 1024 and 4096 are
+    covered elsewhere): initialisation, plain steps and a refresh step, conditionally on the bases."""
+    rank = max(2, min(64, size // 8))
+    count = 3 if size >= 8192 else 5
+    gradients = [oracle.low_rank_plus_noise(size, size, rank, seed=SEED + size + t) for t in range(count)]
+    updates, state, bases = run_recorded(gradients, device, monkeypatch, interval=2, implementation=implementation)
+    assert sorted(bases) == ([0, 2] if count == 3 else [0, 2, 4])
+    assert_conditional_parity(gradients, updates, state, bases, 2, implementation)
+    for side in ("left", "right"):
+        q = state[f"{side}_basis"].double()
+        identity_error = q.T @ q
+        identity_error.diagonal().sub_(1.0)
+        assert identity_error.abs().max().item() <= 1e-4
+
+
 @pytest.mark.parametrize("shape,rank", [((4096, 4096), 64), ((4096, 11008), 128)])
 def test_refresh_factorisation_at_benchmark_sizes(shape, rank, device):
     """P Q, the order and the QR of a refresh, on the state after three Gram updates."""
