@@ -688,6 +688,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 // swapped, D[column][row] += (-X)^T[column][k] V^T[k][row], so that the lanes of a wavefront walk
 // down a column of C and of V (coalesced) and X comes out of LDS.
 constexpr int kPanelApplyCols = 64;
+constexpr int kSliceBatch = 16;  // slices whose loads are in flight together when the slices of V^T [V | C] are summed
 
 // (bx, by) = the workgroup's row block and column group; `col_first` = the first column of C that is
 // updated at all (earlier ones belong to someone else), a multiple of 32.
@@ -706,6 +707,7 @@ __device__ __forceinline__ void panel_apply_tile(const float* __restrict__ part,
   // The tile of C and the rows of V are requested first; they arrive while X is being made.
   const int64_t row_base = (int64_t)bx * 256 + wave * 64;
   const int jr = lane & 31, half = lane >> 5;
+  const T tau_lane = tau[jr];  // (requested with the first loads, not where the substitution needs it)
   Mfma<T>::Acc acc[2][2];
   T vb[2][M / 2];
   // (loads are unconditional: a row past the end reads the last row and is not stored; a column group
@@ -807,7 +809,7 @@ __device__ __forceinline__ void panel_apply_tile(const float* __restrict__ part,
     }
     static_for<0, M>([&](auto step) {
       constexpr int i = decltype(step)::value;
-      const T xi = tau[i] * w[i];
+      const T xi = lane_value<i>(tau_lane) * w[i];
       s_xn[i][lane] = -xi;
       static_for<i + 1, M>([&](auto col) {
         constexpr int l = decltype(col)::value;
@@ -873,6 +875,18 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
                                                             int64_t ldv, int vrow0, float* __restrict__ slices, int nc,
                                                             int64_t slab, PanelCarry carry) {
   using T = float;
+  // Rows of the outer block above this panel: zero in the reflector buffer and in A (the entries of
+  // R there have no reader), so that the block's columns of A hold V in clean form as well.  Nobody
+  // in this launch reads them; the first updating workgroup does it when it has finished (it has time
+  // to spare), the first panel workgroup only when the launch has no updating workgroups.
+  auto zero_above_panel = [&]() {
+    const int above = p - vrow0;
+    for (int col = 0; col < pe - p; ++col)
+      for (int row = threadIdx.x; row < above; row += 256) {
+        vout[row + (int64_t)col * ldv] = T(0);
+        A[(vrow0 + row) + (int64_t)(p + col) * lda] = T(0);
+      }
+  };
   if (carry.slices != nullptr && (int)blockIdx.x < carry.apply_wgs) {
     // ---- the earlier panel's update of the columns behind this panel ----
     const int bx = (int)blockIdx.x % carry.apply_row_blocks, by = (int)blockIdx.x / carry.apply_row_blocks;
@@ -882,6 +896,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     __threadfence();
     __syncthreads();
     if (threadIdx.x == 0) __hip_atomic_fetch_add(carry.done_counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    if (blockIdx.x == 0) zero_above_panel();
     return;
   }
   constexpr int NB = kQrNb, GW = kQrGramWords, XS = NB + 1;
@@ -889,7 +904,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
   __shared__ T s_x[4][64 * XS];  // a wavefront's rows on their way to the MFMA layout, then its Gram matrix
   __shared__ T s_sum[4][NB * NB];  // the wavefronts' parts of a 32 x 32 block of V^T [V | C]
   __shared__ T s_tot[NB * NB];   // s_tot[i * NB + k] = G[i][k], both triangles
-  __shared__ T s_piv[NB * NB];   // s_piv[q * NB + k] = entry k of row p + q
+  __shared__ T s_piv[NB * XS];   // s_piv[q * XS + k] = entry k of row p + q
   __shared__ T s_tc[NB][NB];
   __shared__ T s_scal[NB][2];    // scale, tau of the panel's reflectors
   __shared__ T s_l3[16][16];     // partial sums of the last 16 Gram values, [value][workgroup residue]
@@ -906,28 +921,26 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     s_fail = 0;
     s_seen = T(0);
   }
-  if (wg == 0) {
-    // rows of the outer block above this panel: zero in the reflector buffer and in A (the entries of
-    // R there have no reader), so that the block's columns of A hold V in clean form as well
-    for (int t = tid; t < (p - vrow0) * nbw; t += 256) {
-      const int row = t % (p - vrow0), col = t / (p - vrow0);
-      vout[row + (int64_t)col * ldv] = T(0);
-      A[(vrow0 + row) + (int64_t)(p + col) * lda] = T(0);
-    }
-  }
+  if (wg == 0 && !(carry.slices != nullptr && carry.apply_wgs > 0)) zero_above_panel();
 
   T a[NB];  // a[k] = A[r, p + k]
-  {
-    // (unconditional loads on clamped addresses, zeroed afterwards: tested loads compile to a branch each)
+  // (unconditional loads on clamped addresses, zeroed afterwards by clear_unused: tested loads compile
+  // to a branch each.  The two are separate because the zeroing is the first use of the loaded values:
+  // placed right behind the loads it makes the wavefront wait for them there.)
+  auto load_own_row = [&]() {
     const T* arow = A + (live ? r : n - 1) + (int64_t)p * lda;
 #pragma unroll
-    for (int k = 0; k < NB; ++k) {
-      const T x = arow[(int64_t)min(k, nbw - 1) * lda];
-      a[k] = (live && k < nbw) ? x : T(0);
-    }
-  }
+    for (int k = 0; k < NB; ++k) a[k] = arow[(int64_t)min(k, nbw - 1) * lda];
+  };
+  auto clear_unused = [&]() {
+#pragma unroll
+    for (int k = 0; k < NB; ++k) a[k] = (live && k < nbw) ? a[k] : T(0);
+  };
 
-  if (carry.slices != nullptr) {
+  if (carry.slices == nullptr) {
+    load_own_row();
+    clear_unused();
+  } else {
     // ---- this panel's columns brought up to date with the earlier panel's reflectors ----
     // a[c] -= sum_t V[r][t] X[t][c], X = T^T (V^T C) for the first 32 columns of C, from the slices
     // as in panel_apply_tile: fixed-order sums (16-byte loads), then the forward substitution with
@@ -938,42 +951,42 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     // The product runs on the matrix cores as in panel_apply_tile (operand b = V with lane = row of a
     // 32-row tile, requested now and used after X is known).
     const int jr = lane & 31, half = lane >> 5;
+    // (requested with the first loads: read where the substitution needs it, it would be one more
+    // trip to memory behind the slices)
+    const T tau_lane = carry.tau[jr];
     T vb[2][NB / 2];
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-      const int rl = min(wg * 256 + wave * 64 + rt * 32 + jr, n - 1 - p);  // row of the tile, relative to row p
-      const T* vp = carry.v + rl + (int64_t)half * ldv;
-#pragma unroll
-      for (int ks = 0; ks < NB / 2; ++ks) vb[rt][ks] = vp[(int64_t)(2 * ks) * ldv];
-    }
+    // Order of the requests: the slices first, the reflectors and this thread's own row behind them.
+    // A wavefront can have 63 loads outstanding and they return in order; with the 64 loads of V and
+    // of the row in front, the slices' loads were only issued once those had come back, a second
+    // trip to memory before the sums could start.  V and the row are not needed before the
+    // substitution is over.
     {
       const int eg = 4 * tid;  // entries 4 tid .. 4 tid + 3 of G, and of the first 32 columns of W
-      float4 sg = make_float4(0.f, 0.f, 0.f, 0.f), sw = sg;
+      const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      float4 sg = zero4, sw = zero4;
       auto add4 = [](float4& acc4, const float4& x) {
         acc4.x += x.x;
         acc4.y += x.y;
         acc4.z += x.z;
         acc4.w += x.w;
       };
-      int z = 0;
-      for (; z + 8 <= carry.splits; z += 8) {
-        float4 vg[8], vw[8];
+      // All batches are full: a slice index past the end reads the last slice again and adds zero
+      // (a shorter last batch, or a loop over the remaining slices, would wait for memory once more
+      // per slice).
+      for (int z = 0; z < carry.splits; z += kSliceBatch) {
+        float4 vg[kSliceBatch], vw[kSliceBatch];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const float* base = carry.slices + (int64_t)(z + u) * carry.slab;
+        for (int u = 0; u < kSliceBatch; ++u) {
+          const float* base = carry.slices + (int64_t)min(z + u, carry.splits - 1) * carry.slab;
           vg[u] = *reinterpret_cast<const float4*>(base + eg);
           vw[u] = *reinterpret_cast<const float4*>(base + NB * NB + eg);
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          add4(sg, vg[u]);
-          add4(sw, vw[u]);
+        for (int u = 0; u < kSliceBatch; ++u) {
+          const bool past = z + u >= carry.splits;
+          add4(sg, past ? zero4 : vg[u]);
+          add4(sw, past ? zero4 : vw[u]);
         }
-      }
-      for (; z < carry.splits; ++z) {
-        const float* base = carry.slices + (int64_t)z * carry.slab;
-        add4(sg, *reinterpret_cast<const float4*>(base + eg));
-        add4(sw, *reinterpret_cast<const float4*>(base + NB * NB + eg));
       }
       const int row = eg & (NB - 1), col = eg >> 5;
       s_cg[row][col] = sg.x;
@@ -985,7 +998,15 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       s_cw[col][row + 2] = sw.z;
       s_cw[col][row + 3] = sw.w;
     }
-    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+      const int rl = min(wg * 256 + wave * 64 + rt * 32 + jr, n - 1 - p);  // row of the tile, relative to row p
+      const T* vp = carry.v + rl + (int64_t)half * ldv;
+#pragma unroll
+      for (int ks = 0; ks < NB / 2; ++ks) vb[rt][ks] = vp[(int64_t)(2 * ks) * ldv];
+    }
+    load_own_row();
+    lds_barrier();  // (not __syncthreads(): that would wait for the loads just issued)
     if (wave == 0) {
       T w[NB], gcol[NB];
 #pragma unroll
@@ -995,7 +1016,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       }
       static_for<0, NB>([&](auto step) {
         constexpr int i = decltype(step)::value;
-        const T xi = carry.tau[i] * w[i];
+        const T xi = lane_value<i>(tau_lane) * w[i];
         if (lane < NB) s_cx[i][lane] = -xi;
         static_for<i + 1, NB>([&](auto col) {
           constexpr int l = decltype(col)::value;
@@ -1003,7 +1024,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
         });
       });
     }
-    __syncthreads();
+    lds_barrier();
     {
       // A thread holds its row in a[0..31]; the accumulator layout of a 32 x 32 tile gives lane l
       // columns 8 j + i and lane l + 32 columns 8 j + 4 + i (j, i < 4) of row l.  Swapping the upper
@@ -1033,10 +1054,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
         a[c0 + 4] = __uint_as_float(hi);
       }
     }
-    if (!live) {
-#pragma unroll
-      for (int k = 0; k < NB; ++k) a[k] = T(0);
-    }
+    clear_unused();
   }
 
   int c = 0;  // finished columns
@@ -1044,11 +1062,23 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     const unsigned seq = seq_base + round + 1u;
     unsigned long long* part_c = part + (size_t)(round & 1) * kQrPersistentMaxWg * kQrGramMailWords;
     unsigned long long* piv_c = piv + (round & 1) * NB * NB;
-    // the top block first: it is on its way while the Gram matrix is being computed
+    // What the steps below compare and address with is made opaque once per round.  As loop invariants
+    // the 32 masks `t < nbw`, the 64 masks `r > p + t`, `r == p + t` and the 64 column addresses were
+    // all computed in front of the loop (which usually runs once) and kept in spill lanes and
+    // accumulator registers until their step: 2000 instructions per launch.
+    int nbw_r = nbw, p_r = p, rel_r = wg * 256 + tid;  // (rel_r: this thread's row, counted from row p)
+    int64_t lda_r = lda, ldv_r = ldv;
+    // (the pointers themselves stay as they are: behind an asm statement the compiler no longer knows
+    // that they point to global memory, and its generic stores also count as LDS traffic)
+    asm volatile("" : "+s"(nbw_r), "+s"(p_r), "+s"(lda_r), "+s"(ldv_r));
+    asm volatile("" : "+v"(rel_r));
+    // the top block first: it is on its way while the Gram matrix is being computed (column by column,
+    // 256 contiguous bytes per store instruction: with a row per lane, 32 scattered words each, the
+    // 32 stores took 4 us to issue)
     if (wg == 0 && tid < NB) {
 #pragma unroll
       for (int k = 0; k < NB; ++k)
-        __hip_atomic_store(piv_c + tid * NB + k, mailbox_pack(live ? a[k] : T(0), seq), __ATOMIC_RELAXED,
+        __hip_atomic_store(piv_c + k * NB + tid, mailbox_pack(live ? a[k] : T(0), seq), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
     // Gram matrix of this wavefront's hidden rows (finished columns ride along; nobody reads them)
@@ -1056,7 +1086,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       T* xs = s_x[wave];
 #pragma unroll
       for (int k = 0; k < NB; ++k) xs[lane * XS + k] = hidden ? a[k] : T(0);
-      __syncthreads();
+      lds_barrier();  // (the barriers of this loop order LDS traffic only; __syncthreads() would also wait for the mailbox stores)
       Mfma<T>::Acc acc = {}, acc_odd = {};  // two chains, so that an instruction need not wait for the one before it
 #pragma unroll
       for (int s = 0; s < 32; s += 2) {
@@ -1070,7 +1100,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
 #pragma unroll
       for (int v = 0; v < Mfma<T>::NACC; ++v) xs[Mfma<T>::acc_row(v, lane) * NB + (lane & 31)] = acc[v];
     }
-    __syncthreads();
+    lds_barrier();
     for (int idx = tid; idx < GW; idx += 256) {
       int i, k;
       gram_unpack_index(idx, i, k);
@@ -1116,14 +1146,14 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
         for (int u = 0; u < 4; ++u) slot[u] = piv_c + tid + 256 * u;
         ok = mailbox_wait<4>(slot, used, seq, error, spin_limit, v);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) s_piv[tid + 256 * u] = v[u];
+        for (int u = 0; u < 4; ++u) s_piv[(tid & (NB - 1)) * XS + (tid >> 5) + 8 * u] = v[u];  // word k * NB + q of the mail
       }
       if (!ok) {
         __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_fail = 1;
       }
     }
-    __syncthreads();
+    lds_barrier();
     if (s_fail) return;
     if (tid < 16) {
       T total = T(0);
@@ -1134,7 +1164,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       s_tot[i * NB + k] = total;
       s_tot[k * NB + i] = total;
     }
-    __syncthreads();
+    lds_barrier();
     if (wave == 0) {
       // Lanes 0..31 hold the top block E, lanes 32..63 the Gram matrix G: lane k of either half owns
       // column k of its matrix (x[q] = entry q).  A step needs entry q of column t of E in every lane
@@ -1148,7 +1178,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       const bool upper = lane >= NB;
       T x[NB];
 #pragma unroll
-      for (int q = 0; q < NB; ++q) x[q] = upper ? s_tot[q * NB + k] : s_piv[q * NB + k];
+      for (int q = 0; q < NB; ++q) x[q] = upper ? s_tot[q * NB + k] : s_piv[q * XS + k];
       T size_diag = fabsf(s_tot[k * NB + k]);  // size of the terms G[k][k] is made of (same in both halves)
       T seen = s_seen;
       int done = c;
@@ -1158,7 +1188,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       // and the next round starts from their rows.
       static_for<0, NB>([&](auto step) {
         constexpr int t = decltype(step)::value;
-        if (t >= c && t < nbw) {
+        if (t >= c && t < nbw_r) {
           // (the lane's column number and half are made opaque per step: otherwise the compiler keeps
           // the 32 masks `k > t` and the half masks live across the whole panel in scalar registers it
           // does not have, and reloads each from a spill slot with two cross-lane reads)
@@ -1200,7 +1230,7 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
           const T x2_explicit = lane_value<t>(ek);
           const T size_t_ = lane_value<t>(size_diag);
           // (the last column of the matrix has nothing below its pivot: exactly zero, so tau = 0 as in LAPACK)
-          const T x2 = (p + t < n - 1) ? x2_explicit + fmaxf(hidden2, T(0)) : T(0);
+          const T x2 = (p_r + t < n - 1) ? x2_explicit + fmaxf(hidden2, T(0)) : T(0);
           const bool finite = hidden2 - hidden2 == T(0);
           open = open && (t == c || (finite && alpha * alpha + x2 >= kQrRoundGuard * size_t_));
           const Reflector h = make_reflector_fast(alpha, x2, kQrNegligible * seen);
@@ -1228,28 +1258,57 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
         s_seen = seen;
       }
     }
-    __syncthreads();
+    lds_barrier();
     const int done = s_done;
-    static_for<0, NB>([&](auto step) {
+    // The rows' owners apply the steps [c, done).  One instruction stream for the rows below the pivot
+    // (v = scaled entry), the pivot row (v = 1) and the finished rows above it (v = 0); the finished
+    // column's register then holds this row of V (nothing reads it before the end).  The usual case,
+    // a whole panel in one round, runs without a test per step, so that the coefficients of the next
+    // step are on their way from LDS while this one is applied; nothing is stored before all steps
+    // are done.
+    auto apply_step = [&](auto step) {
       constexpr int t = decltype(step)::value;
-      if (t >= c && t < done) {
-        const T scale = s_scal[t][0];
-        const int jt = p + t;
-        // one instruction stream for the rows below the pivot (v = scaled entry), the pivot row
-        // (v = 1) and the finished rows above it (v = 0)
-        const bool below = r > jt, pivot = r == jt;
-        const T v = below ? a[t] * scale : (pivot ? T(1) : T(0));
+      const T scale = s_scal[t][0];
+      const bool below = rel_r > t, pivot = rel_r == t;
+      const T v = below ? a[t] * scale : (pivot ? T(1) : T(0));
 #pragma unroll
-        for (int k = t + 1; k < NB; ++k) a[k] -= s_tc[t][k] * v;
-        if (live && pivot) tau[jt] = s_scal[t][1];
-        if (live) {
-          // clean form in both copies, as in the kernel above
-          A[r + (int64_t)jt * lda] = v;
-          vout[(r - vrow0) + (int64_t)t * ldv] = v;
+      for (int k = t + 1; k < NB; ++k) a[k] -= s_tc[t][k] * v;
+      a[t] = v;
+    };
+    const bool whole = c == 0 && done == NB;
+    if (whole) {
+      static_for<0, NB>(apply_step);
+    } else {
+      static_for<0, NB>([&](auto step) {
+        constexpr int t = decltype(step)::value;
+        if (t >= c && t < done) apply_step(step);
+      });
+    }
+    if (wg == 0 && tid < NB && tid >= c && tid < done && live) tau[p_r + tid] = s_scal[tid][1];
+    if (live) {
+      // clean form in both copies, as in the kernel above; the addresses walk from column to column
+      T* acol = A + r + (int64_t)p_r * lda_r;
+      T* vcol = vout + (r - vrow0);
+      if (whole) {
+#pragma unroll
+        for (int t = 0; t < NB; ++t) {
+          *acol = a[t];
+          *vcol = a[t];
+          acol += lda_r;
+          vcol += ldv_r;
         }
-        a[t] = v;  // the finished column's register now holds this row of V (nothing reads it before the end)
+      } else {
+        static_for<0, NB>([&](auto step) {
+          constexpr int t = decltype(step)::value;
+          if (t >= c && t < done) {
+            *acol = a[t];
+            *vcol = a[t];
+          }
+          acol += lda_r;
+          vcol += ldv_r;
+        });
       }
-    });
+    }
     c = done;
   }
   if (slices == nullptr) return;
