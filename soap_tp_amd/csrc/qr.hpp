@@ -1017,11 +1017,15 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       static_for<0, NB>([&](auto step) {
         constexpr int i = decltype(step)::value;
         const T xi = lane_value<i>(tau_lane) * w[i];
-        if (lane < NB) s_cx[i][lane] = -xi;
+        s_cx[i][lane & (NB - 1)] = -xi;  // (both halves of the wavefront hold the same 32 columns)
         static_for<i + 1, NB>([&](auto col) {
           constexpr int l = decltype(col)::value;
           w[l] -= lane_value<l>(gcol[i]) * xi;
         });
+        // (the updates of a step stay in that step: left to itself the compiler gathers all updates
+        // of one w[l] into a chain in front of its use and reads the 496 entries of G ahead, through
+        // more scalar registers than there are)
+        static_for<i + 1, NB>([&](auto col) { keep_behind_wait(w[decltype(col)::value]); });
       });
     }
     lds_barrier();
