@@ -273,13 +273,18 @@ __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&s
 // not, so all must be valid memory: the addresses are then constant offsets from two bases, which
 // keeps this many loads in flight within the register budget).  False after too many polls or once
 // the error flag is up.
-template <int COUNT, int STRIDE, int EXTRA, int STRIDE3>
+// With TOP = 4 the same trip also fetches the words top[0], top[256], top[512], top[768] (values in
+// top_value); with TOP = 0 `top` and `top_value` are not touched.
+template <int COUNT, int STRIDE, int EXTRA, int STRIDE3, int TOP = 0>
 __device__ __forceinline__ bool mailbox_wait_sum(const unsigned long long* base, int count,
                                                  const unsigned long long* base3, int count3, unsigned seq,
-                                                 const int* error, unsigned spin_limit, float& sum, float& sum3) {
+                                                 const int* error, unsigned spin_limit, float& sum, float& sum3,
+                                                 const unsigned long long* top = nullptr, float* top_value = nullptr) {
   unsigned spins = 0;
   for (;;) {
-    unsigned long long word[COUNT + EXTRA];
+    unsigned long long word[COUNT + EXTRA], top_word[TOP > 0 ? TOP : 1];
+#pragma unroll
+    for (int u = 0; u < TOP; ++u) top_word[u] = __hip_atomic_load(top + 256 * u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int u = 0; u < COUNT; ++u)
       word[u] = __hip_atomic_load(base + u * STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -291,11 +296,65 @@ __device__ __forceinline__ bool mailbox_wait_sum(const unsigned long long* base,
     for (int u = 0; u < COUNT; ++u) ready = ready && (u >= count || (unsigned)(word[u] >> 32) == seq);
 #pragma unroll
     for (int u = 0; u < EXTRA; ++u) ready = ready && (u >= count3 || (unsigned)(word[COUNT + u] >> 32) == seq);
+#pragma unroll
+    for (int u = 0; u < TOP; ++u) ready = ready && (unsigned)(top_word[u] >> 32) == seq;
     if (ready) {
+#pragma unroll
+      for (int u = 0; u < TOP; ++u) top_value[u] = __uint_as_float((unsigned)top_word[u]);
 #pragma unroll
       for (int u = 0; u < COUNT; ++u) sum += (u < count) ? __uint_as_float((unsigned)word[u]) : 0.0f;
 #pragma unroll
       for (int u = 0; u < EXTRA; ++u) sum3 += (u < count3) ? __uint_as_float((unsigned)word[COUNT + u]) : 0.0f;
+      return true;
+    }
+    ++spins;
+    if (spins > spin_limit) return false;
+    if ((spins & 63u) == 0 && __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
+// Everything a thread of the whole-panel kernel needs from an exchange, in one trip to memory, for
+// launches of at most COUNT workgroups: its two Gram values from all workgroups (base0, base1,
+// stride 64 words per workgroup), its share of the last sixteen values (base3, stride 16 x 64 words,
+// `count3` <= EXTRA of them) and its four words of the top block.  The sums run over the workgroups
+// in ascending order.  Every slot is loaded whether it counts or not.  False after too many polls
+// or once the error flag is up.
+template <int COUNT, int EXTRA>
+__device__ __forceinline__ bool mailbox_wait_all(const unsigned long long* base0, const unsigned long long* base1,
+                                                 int count, const unsigned long long* base3, int count3,
+                                                 const unsigned long long* top, unsigned seq, const int* error,
+                                                 unsigned spin_limit, float& sum0, float& sum1, float& sum3,
+                                                 float (&top_value)[4]) {
+  unsigned spins = 0;
+  for (;;) {
+    unsigned long long w0[COUNT], w1[COUNT], w3[EXTRA], wt[4];
+#pragma unroll
+    for (int u = 0; u < COUNT; ++u) w0[u] = __hip_atomic_load(base0 + u * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int u = 0; u < COUNT; ++u) w1[u] = __hip_atomic_load(base1 + u * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int u = 0; u < EXTRA; ++u)
+      w3[u] = __hip_atomic_load(base3 + u * 16 * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) wt[u] = __hip_atomic_load(top + 256 * u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool ready = true;
+#pragma unroll
+    for (int u = 0; u < COUNT; ++u)
+      ready = ready && (u >= count || ((unsigned)(w0[u] >> 32) == seq && (unsigned)(w1[u] >> 32) == seq));
+#pragma unroll
+    for (int u = 0; u < EXTRA; ++u) ready = ready && (u >= count3 || (unsigned)(w3[u] >> 32) == seq);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) ready = ready && (unsigned)(wt[u] >> 32) == seq;
+    if (ready) {
+#pragma unroll
+      for (int u = 0; u < COUNT; ++u) sum0 += (u < count) ? __uint_as_float((unsigned)w0[u]) : 0.0f;
+#pragma unroll
+      for (int u = 0; u < COUNT; ++u) sum1 += (u < count) ? __uint_as_float((unsigned)w1[u]) : 0.0f;
+#pragma unroll
+      for (int u = 0; u < EXTRA; ++u) sum3 += (u < count3) ? __uint_as_float((unsigned)w3[u]) : 0.0f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) top_value[u] = __uint_as_float((unsigned)wt[u]);
       return true;
     }
     ++spins;
@@ -1123,35 +1182,46 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       T sum[2] = {T(0), T(0)}, sum3 = T(0);
       const unsigned long long* base3 = part_c + gram_mail_offset(512 + (tid & 15), tid >> 4);
       const int count3 = (nwg - (tid >> 4) + 15) >> 4;  // workgroups tid / 16, tid / 16 + 16, ... below nwg
+      float top_value[4] = {0.f, 0.f, 0.f, 0.f};
+      if (nwg <= 32) {
+        // one trip to memory for the lot (three in the general form below: the two values one after
+        // the other, then the top block; with more than 32 workgroups, where a thread has over a
+        // hundred loads to make either way, the single trip was no faster)
+        const unsigned long long* base0 = part_c + gram_mail_offset(tid, 0);
+        const unsigned long long* base1 = part_c + gram_mail_offset(tid + 256, 0);
+        if (nwg <= 16)
+          ok = mailbox_wait_all<16, 1>(base0, base1, nwg, base3, count3, piv_c + tid, seq, error, spin_limit, sum[0], sum[1],
+                                       sum3, top_value);
+        else
+          ok = mailbox_wait_all<32, 2>(base0, base1, nwg, base3, count3, piv_c + tid, seq, error, spin_limit, sum[0], sum[1],
+                                       sum3, top_value);
+      } else {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int idx = tid + 256 * half;
+          for (int w0 = 0; w0 < nwg && ok; w0 += BATCH) {
+            // (the last batch may reach past workgroup 127: the buffer has BATCH spare rows)
+            const unsigned long long* base = part_c + gram_mail_offset(idx, w0);
+            T unused = T(0);
+            if (half == 1 && w0 == 0)  // (the last sixteen values and the top block ride along with this trip)
+              ok = mailbox_wait_sum<BATCH, 64, L3, 16 * 64, 4>(base, nwg - w0, base3, count3, seq, error, spin_limit,
+                                                               sum[half], sum3, piv_c + tid, top_value);
+            else
+              ok = mailbox_wait_sum<BATCH, 64, 0, 1>(base, nwg - w0, base, 0, seq, error, spin_limit, sum[half], unused);
+          }
+        }
+      }
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const int idx = tid + 256 * half;
-        for (int w0 = 0; w0 < nwg && ok; w0 += BATCH) {
-          // (the last batch may reach past workgroup 127: the buffer has BATCH spare rows)
-          const unsigned long long* base = part_c + gram_mail_offset(idx, w0);
-          T unused = T(0);
-          if (half == 1 && w0 == 0)
-            ok = mailbox_wait_sum<BATCH, 64, L3, 16 * 64>(base, nwg - w0, base3, count3, seq, error, spin_limit, sum[half],
-                                                          sum3);
-          else
-            ok = mailbox_wait_sum<BATCH, 64, 0, 1>(base, nwg - w0, base, 0, seq, error, spin_limit, sum[half], unused);
-        }
         int i, k;
-        gram_unpack_index(idx, i, k);
+        gram_unpack_index(tid + 256 * half, i, k);
         s_tot[i * NB + k] = sum[half];
         s_tot[k * NB + i] = sum[half];
       }
       s_l3[tid & 15][tid >> 4] = sum3;
-      if (ok) {
-        const unsigned long long* slot[4];
-        const bool used[4] = {true, true, true, true};
-        float v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) slot[u] = piv_c + tid + 256 * u;
-        ok = mailbox_wait<4>(slot, used, seq, error, spin_limit, v);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) s_piv[(tid & (NB - 1)) * XS + (tid >> 5) + 8 * u] = v[u];  // word k * NB + q of the mail
-      }
+      for (int u = 0; u < 4; ++u)
+        s_piv[(tid & (NB - 1)) * XS + (tid >> 5) + 8 * u] = top_value[u];  // word k * NB + q of the mail
       if (!ok) {
         __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_fail = 1;
