@@ -273,18 +273,13 @@ __device__ __forceinline__ bool mailbox_wait(const unsigned long long* const (&s
 // not, so all must be valid memory: the addresses are then constant offsets from two bases, which
 // keeps this many loads in flight within the register budget).  False after too many polls or once
 // the error flag is up.
-// With TOP = 4 the same trip also fetches the words top[0], top[256], top[512], top[768] (values in
-// top_value); with TOP = 0 `top` and `top_value` are not touched.
-template <int COUNT, int STRIDE, int EXTRA, int STRIDE3, int TOP = 0>
+template <int COUNT, int STRIDE, int EXTRA, int STRIDE3>
 __device__ __forceinline__ bool mailbox_wait_sum(const unsigned long long* base, int count,
                                                  const unsigned long long* base3, int count3, unsigned seq,
-                                                 const int* error, unsigned spin_limit, float& sum, float& sum3,
-                                                 const unsigned long long* top = nullptr, float* top_value = nullptr) {
+                                                 const int* error, unsigned spin_limit, float& sum, float& sum3) {
   unsigned spins = 0;
   for (;;) {
-    unsigned long long word[COUNT + EXTRA], top_word[TOP > 0 ? TOP : 1];
-#pragma unroll
-    for (int u = 0; u < TOP; ++u) top_word[u] = __hip_atomic_load(top + 256 * u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned long long word[COUNT + EXTRA];
 #pragma unroll
     for (int u = 0; u < COUNT; ++u)
       word[u] = __hip_atomic_load(base + u * STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -296,11 +291,7 @@ __device__ __forceinline__ bool mailbox_wait_sum(const unsigned long long* base,
     for (int u = 0; u < COUNT; ++u) ready = ready && (u >= count || (unsigned)(word[u] >> 32) == seq);
 #pragma unroll
     for (int u = 0; u < EXTRA; ++u) ready = ready && (u >= count3 || (unsigned)(word[COUNT + u] >> 32) == seq);
-#pragma unroll
-    for (int u = 0; u < TOP; ++u) ready = ready && (unsigned)(top_word[u] >> 32) == seq;
     if (ready) {
-#pragma unroll
-      for (int u = 0; u < TOP; ++u) top_value[u] = __uint_as_float((unsigned)top_word[u]);
 #pragma unroll
       for (int u = 0; u < COUNT; ++u) sum += (u < count) ? __uint_as_float((unsigned)word[u]) : 0.0f;
 #pragma unroll
@@ -1173,12 +1164,10 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
                          __HIP_MEMORY_SCOPE_AGENT);
     }
     {
-      // Fixed-order sums over the workgroups.  Thread tid takes the values tid and tid + 256 over all
-      // workgroups (48 loads in flight, so one trip each up to 48 workgroups); the 16 values from 512
-      // on are split sixteen ways over the workgroups (thread tid: value 512 + tid % 16, workgroups
-      // tid / 16, tid / 16 + 16, ...) and ride along with the second trip.
+      // Fixed-order sums over the workgroups.  Up to 32 workgroups thread tid takes the values tid and
+      // tid + 256 over all workgroups; the 16 values from 512 on are split sixteen ways over the
+      // workgroups (thread tid: value 512 + tid % 16, workgroups tid / 16, tid / 16 + 16, ...).
       bool ok = true;
-      constexpr int L3 = kQrPersistentMaxWg / 16, BATCH = 48;  // BATCH * 64 = the spare words behind the buffer
       T sum[2] = {T(0), T(0)}, sum3 = T(0);
       const unsigned long long* base3 = part_c + gram_mail_offset(512 + (tid & 15), tid >> 4);
       const int count3 = (nwg - (tid >> 4) + 15) >> 4;  // workgroups tid / 16, tid / 16 + 16, ... below nwg
@@ -1196,19 +1185,37 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
           ok = mailbox_wait_all<32, 2>(base0, base1, nwg, base3, count3, piv_c + tid, seq, error, spin_limit, sum[0], sum[1],
                                        sum3, top_value);
       } else {
+        // More workgroups: two levels.  All-to-all, every workgroup would read the 528 values of every
+        // other one (8 MB per exchange at 43 workgroups, 10 us on the fabric between the XCDs).
+        // Level 1: this workgroup sums its share of the values, `per` consecutive ones, over all
+        // workgroups (one thread per value, workgroups in ascending order) and publishes the totals;
+        // level 2: every thread fetches the totals it needs, and its words of the top block.
+        const int per = (GW + nwg - 1) / nwg;  // (at most 16)
+        unsigned long long* total_c =
+            part + (size_t)2 * kQrPersistentMaxWg * kQrGramMailWords + (size_t)(round & 1) * kQrGramMailWords;
+        const int mine = wg * per + tid;
+        if (tid < per && mine < GW) {
+          T total = T(0), unused = T(0);
+          for (int w0 = 0; w0 < nwg && ok; w0 += 32)  // (a batch may reach past the last workgroup: spare rows)
+            ok = mailbox_wait_sum<32, 64, 0, 1>(part_c + gram_mail_offset(mine, w0), nwg - w0, part_c, 0, seq, error,
+                                                spin_limit, total, unused);
+          if (ok) __hip_atomic_store(total_c + mine, mailbox_pack(total, seq), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (ok) {
+          const unsigned long long* slot[7];
+          const bool used[7] = {true, true, true, true, true, true, true};
+          float v[7];
+          slot[0] = total_c + tid;
+          slot[1] = total_c + 256 + tid;
+          slot[2] = total_c + 512 + (tid & 15);
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int idx = tid + 256 * half;
-          for (int w0 = 0; w0 < nwg && ok; w0 += BATCH) {
-            // (the last batch may reach past workgroup 127: the buffer has BATCH spare rows)
-            const unsigned long long* base = part_c + gram_mail_offset(idx, w0);
-            T unused = T(0);
-            if (half == 1 && w0 == 0)  // (the last sixteen values and the top block ride along with this trip)
-              ok = mailbox_wait_sum<BATCH, 64, L3, 16 * 64, 4>(base, nwg - w0, base3, count3, seq, error, spin_limit,
-                                                               sum[half], sum3, piv_c + tid, top_value);
-            else
-              ok = mailbox_wait_sum<BATCH, 64, 0, 1>(base, nwg - w0, base, 0, seq, error, spin_limit, sum[half], unused);
-          }
+          for (int u = 0; u < 4; ++u) slot[3 + u] = piv_c + tid + 256 * u;
+          ok = mailbox_wait<7>(slot, used, seq, error, spin_limit, v);
+          sum[0] = v[0];
+          sum[1] = v[1];
+          sum3 = (tid < 16) ? v[2] : T(0);  // (s_l3 holds sixteen partial sums per value: here one of them is the total)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) top_value[u] = v[3 + u];
         }
       }
 #pragma unroll
@@ -1425,18 +1432,23 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     // past the end the last column): such rows have V = 0 and such columns are not stored.  The
     // column's base address is the same for all lanes, the row a 32-bit index.
     const int rr = live ? r : n - 1;
-    T cur[NB];
-    auto load_block = [&](int c0) {
+    // Two blocks of C are on their way at any time (block jb covers columns 32 (jb - 1) ...): the
+    // matrix was just written by other workgroups, so a block's loads come from memory, which takes
+    // longer than the products of one block.
+    T cur[2][NB];
+    auto load_block = [&](T (&dst)[NB], int jb) {
+      const int c0 = (jb - 1) * NB;
       const T* base = A + (int64_t)(pe + c0) * lda;
       if (c0 + NB <= nc) {
 #pragma unroll
-        for (int k = 0; k < NB; ++k) cur[k] = base[(int64_t)k * lda + rr];
+        for (int k = 0; k < NB; ++k) dst[k] = base[(int64_t)k * lda + rr];
       } else {
 #pragma unroll
-        for (int k = 0; k < NB; ++k) cur[k] = base[(int64_t)min(k, nc - 1 - c0) * lda + rr];
+        for (int k = 0; k < NB; ++k) dst[k] = base[(int64_t)min(k, nc - 1 - c0) * lda + rr];
       }
     };
-    if (blocks > 1) load_block(0);  // on its way while V is staged and V^T V computed
+    if (blocks > 1) load_block(cur[0], 1);  // on their way while V is staged and V^T V computed
+    if (blocks > 2) load_block(cur[1], 2);
 #pragma unroll
     for (int k = 0; k < NB; ++k) xs[lane * XS + k] = a[k];
     T vb[NB];
@@ -1464,11 +1476,11 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       acc += acc_odd;
       emit(0, acc);
     }
-    for (int jb = 1; jb < blocks; ++jb) {
+    auto multiply_block = [&](T (&src)[NB], int jb) {
       // (a wavefront's LDS accesses complete in order: the reads of the block before are done)
 #pragma unroll
-      for (int k = 0; k < NB; ++k) xs[lane * XS + k] = cur[k];
-      if (jb + 1 < blocks) load_block(jb * NB);  // the next block's loads are in flight during this block's products
+      for (int k = 0; k < NB; ++k) xs[lane * XS + k] = src[k];
+      if (jb + 2 < blocks) load_block(src, jb + 2);  // into the registers just emptied
       T x[NB];
 #pragma unroll
       for (int s = 0; s < NB; ++s) x[s] = xs[(2 * s + half) * XS + l31];
@@ -1480,6 +1492,10 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
       }
       acc += acc_odd;
       emit(jb, acc);
+    };
+    for (int jb = 1; jb < blocks; jb += 2) {
+      multiply_block(cur[0], jb);
+      if (jb + 1 < blocks) multiply_block(cur[1], jb + 1);
     }
   }
 }
@@ -1914,7 +1930,9 @@ static inline void launch_extract_v(hipStream_t s, const T* A, int64_t lda, int 
 // kernels use (four columns per round: 4 x 32 and 4 x 32; whole panel: 9 x 64 and 32 x 32).
 constexpr int kQrMailWords = kQrGramMailWords > kQrRoundMax * kQrNb ? kQrGramMailWords : kQrRoundMax * kQrNb;
 constexpr int kQrMailPivotWords = kQrNb * kQrNb;
-constexpr int kQrMailSpareWords = 48 * 64;  // the whole-panel kernel loads rows of 48 workgroups at a time, used or not
+// behind the mailboxes: the totals of the whole-panel kernel's two-level exchange (2 x 576 words), and room
+// for its batched loads, which read up to 31 rows past the last workgroup, used or not
+constexpr int kQrMailSpareWords = 48 * 64;
 constexpr int kQrWholePanel = kQrNb;  // columns_per_round value that selects qr_panel_gram_kernel
 
 template <typename T>
