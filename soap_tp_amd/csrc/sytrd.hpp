@@ -189,6 +189,7 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
   __shared__ T s_t4[4][2 * NB];
   __shared__ T s_wj[NB], s_vj[NB];
   __shared__ T s_red[4][2 * NB];
+  __shared__ T s_row[2 * NB];  // row jn + 1 of [W | Vc] (columns up to i), written by its owner in workgroup 0
   __shared__ T s_w4[4];
   __shared__ T s_x;
   __shared__ int s_fail;
@@ -207,6 +208,7 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
   for (int k = 0; k < NB; ++k) vr[k] = wr[k] = T(0);
   T vi = T(0), wv = T(0);  // this row of column i: v_j and the unfinished w_j
   T alpha2 = T(0), w_jn_i = T(0);
+  T acc_old = T(0), a_loaded = T(0);
 
   if (do_d) {
     // ---- D(j): w = tau (y - V (W^T v) - W (V^T v)) ----
@@ -251,10 +253,23 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
     }
     if (tid == 0) mail_post(mail_dot + 2 * wg, dot, seq);
     if (r == jn) mail_post(mail_dot + 2 * kTrdMaxWg, wv, seq);  // the unfinished W[jn, i]
+    // While the messages travel: what the finished columns k < i contribute to the update of column
+    // jn (row jn of those columns is final in memory), and column jn itself.
+    if (tid < i) {
+      s_wj[tid] = W[jn + (int64_t)tid * ldw];
+      s_vj[tid] = Vc[jn + (int64_t)tid * ldw];
+    }
+    if (live) a_loaded = A[r + (int64_t)jn * lda];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < NB; ++k)
+      if (k < i) acc_old += vr[k] * s_wj[k] + wr[k] * s_vj[k];
     T total, w_jn_raw;
     if (!mail_gather<T>(mail_dot, nwg, seq, error, spin_limit, s_w4, &s_x, &s_fail, &total, &w_jn_raw)) return;
     alpha2 = T(-0.5) * tau[j] * total;
     w_jn_i = w_jn_raw + alpha2;  // v_j has its unit entry in row jn
+  } else if (live) {
+    a_loaded = A[r + (int64_t)jn * lda];
   }
 
   // ---- A(jn): finish w_j, bring column jn up to date, norm of its sub-column ----
@@ -263,21 +278,13 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
   if (do_d) {
     wf = wv + alpha2 * vi;
     if (live) W[r + (int64_t)i * ldw] = wf;
-    if (tid < i) {  // row jn of the finished columns
-      s_wj[tid] = W[jn + (int64_t)tid * ldw];
-      s_vj[tid] = Vc[jn + (int64_t)tid * ldw];
-    }
-    __syncthreads();
   }
   T a = T(0), x2 = T(0);
   if (live) {
-    a = A[r + (int64_t)jn * lda];
+    a = a_loaded;
     if (do_d) {
-      T acc = vi * w_jn_i + wf;  // column i: Vc[r,i] W[jn,i] + W[r,i] Vc[jn,i], Vc[jn,i] = 1
-#pragma unroll
-      for (int k = 0; k < NB; ++k)
-        if (k < i) acc += vr[k] * s_wj[k] + wr[k] * s_vj[k];
-      a -= acc;
+      // column i: Vc[r,i] W[jn,i] + W[r,i] Vc[jn,i], Vc[jn,i] = 1
+      a -= (vi * w_jn_i + wf) + acc_old;
       A[r + (int64_t)jn * lda] = a;
     }
     if (r == jn) d[jn] = a;
@@ -287,6 +294,30 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
   const T norm_part = block_sum_shuffle(x2, s_w4);
   if (tid == 0) mail_post(mail_norm + 2 * wg, norm_part, seq);
   if (r == jn + 1) mail_post(mail_norm + 2 * kTrdMaxWg, a, seq);  // alpha
+  // While the messages travel: v = scale * a below row jn + 1, so this workgroup's part of W^T v
+  // and V^T v is scale times its part of W^T a and V^T a over those rows, plus row jn + 1 itself
+  // (where v = 1); the sums over the rows are formed now and scaled once `scale` is known.
+  {
+    const T u = (live && r > jn + 1) ? a : T(0);
+    T pw[NB], pv[NB];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      const T wk = (do_d && k == i) ? wf : wr[k];  // wr, vr are zero beyond column i
+      const T vk = (do_d && k == i) ? vi : vr[k];
+      pw[k] = wk * u;
+      pv[k] = vk * u;
+      if (r == jn + 1) {  // (one thread of workgroup 0)
+        s_row[k] = wk;
+        s_row[NB + k] = vk;
+      }
+    }
+    const T tw = wave_reduce_32<T>(pw, lane);
+    const T tv = wave_reduce_32<T>(pv, lane);
+    if ((lane & 1) == 0) {
+      s_red[wave][(lane >> 1) & 31] = tw;
+      s_red[wave][NB + ((lane >> 1) & 31)] = tv;
+    }
+  }
   T x2_total, alpha;
   if (!mail_gather<T>(mail_norm, nwg, seq, error, spin_limit, s_w4, &s_x, &s_fail, &x2_total, &alpha)) return;
 
@@ -319,25 +350,12 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
       Vc2[rr + (int64_t)in * ldw] = T(0);
     }
   }
-  {
-    T pw[NB], pv[NB];
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {
-      const T wk = (do_d && k == i) ? wf : wr[k];  // wr, vr are zero beyond column i
-      const T vk = (do_d && k == i) ? vi : vr[k];
-      pw[k] = wk * v;
-      pv[k] = vk * v;
-    }
-    const T tw = wave_reduce_32<T>(pw, lane);
-    const T tv = wave_reduce_32<T>(pv, lane);
-    if ((lane & 1) == 0) {
-      s_red[wave][(lane >> 1) & 31] = tw;
-      s_red[wave][NB + ((lane >> 1) & 31)] = tv;
-    }
+  // (s_red and s_row were written before the wait; the barriers of mail_gather lie in between)
+  if (tid < 2 * NB) {
+    const T below = (s_red[0][tid] + s_red[1][tid]) + (s_red[2][tid] + s_red[3][tid]);
+    const bool has_row = wg == 0 && jn + 1 < n;  // row jn + 1 is row 1 of workgroup 0
+    t_part[(int64_t)wg * 2 * NB + tid] = scale * below + (has_row ? s_row[tid] : T(0));
   }
-  __syncthreads();
-  if (tid < 2 * NB)
-    t_part[(int64_t)wg * 2 * NB + tid] = (s_red[0][tid] + s_red[1][tid]) + (s_red[2][tid] + s_red[3][tid]);
 }
 
 // Kernel C.  The trailing matrix (rows and columns o = j+1 .. n-1, only its lower triangle is
