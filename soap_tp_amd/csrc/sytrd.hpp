@@ -81,12 +81,25 @@ __device__ __forceinline__ T reduce_partials(const T* __restrict__ part, int cou
   return block_sum_256(s, red);
 }
 
-// Sum over the 256 threads of a workgroup: xor-shuffles inside each wavefront, then the four
-// wavefront sums in a fixed order.  `s_w` is 4 values of shared memory; two barriers.
+// Sum over the wavefront, in every lane: four steps inside the 16-lane rows on data-parallel-primitive
+// moves (partners lane ^ 1, ^ 2, ^ 7, ^ 15), then the rows 16 and 32 lanes apart on the lane-swap
+// instructions.  (Six xor-shuffles take six trips through the LDS crossbar, two each for a double.)
+template <typename T>
+__device__ __forceinline__ T wave_sum_all(T v) {
+  v += dpp_partner<kDppQuadXor1>(v);
+  v += dpp_partner<kDppQuadXor2>(v);
+  v += dpp_partner<kDppRowHalfMirror>(v);
+  v += dpp_partner<kDppRowMirror>(v);
+  v = swap_add<false>(v, v);
+  v = swap_add<true>(v, v);
+  return v;
+}
+
+// Sum over the 256 threads of a workgroup: each wavefront's sum, then the four wavefront sums in a
+// fixed order.  `s_w` is 4 values of shared memory; two barriers.
 template <typename T>
 __device__ __forceinline__ T block_sum_shuffle(T v, T* s_w) {
-#pragma unroll
-  for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m, 64);
+  v = wave_sum_all(v);
   __syncthreads();  // earlier readers of s_w are done
   if ((threadIdx.x & 63) == 0) s_w[threadIdx.x >> 6] = v;
   __syncthreads();
@@ -212,6 +225,24 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
 
   if (do_d) {
     // ---- D(j): w = tau (y - V (W^T v) - W (V^T v)) ----
+    // This row of the panel's finished columns and of y first: the loads are on their way while the
+    // partial products of the launch before are summed.
+    T y = T(0);
+    if (live) {
+#pragma unroll
+      for (int k = 0; k < NB; ++k) {
+        vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
+        wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
+      }
+      vi = Vc[r + (int64_t)i * ldw];
+      for (int c0 = 0; c0 < n_slots; c0 += 32) {  // 32 slot loads in flight, summed in slot order
+        T yp[32];
+#pragma unroll
+        for (int c = 0; c < 32; ++c) yp[c] = (c0 + c < n_slots) ? y_part[(int64_t)(c0 + c) * n + r] : T(0);
+#pragma unroll
+        for (int c = 0; c < 32; ++c) y += yp[c];
+      }
+    }
     {
       // 2*NB columns x n_t_part partials: 4 strided partial sums per column, then 4 adds
       const int c = tid & (2 * NB - 1), g0 = tid >> 6;
@@ -225,20 +256,6 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
     __syncthreads();
     T prod = T(0);
     if (live) {
-#pragma unroll
-      for (int k = 0; k < NB; ++k) {
-        vr[k] = (k < i) ? Vc[r + (int64_t)k * ldw] : T(0);
-        wr[k] = (k < i) ? W[r + (int64_t)k * ldw] : T(0);
-      }
-      vi = Vc[r + (int64_t)i * ldw];
-      T y = T(0);
-      for (int c0 = 0; c0 < n_slots; c0 += 32) {  // 32 slot loads in flight, summed in slot order
-        T yp[32];
-#pragma unroll
-        for (int c = 0; c < 32; ++c) yp[c] = (c0 + c < n_slots) ? y_part[(int64_t)(c0 + c) * n + r] : T(0);
-#pragma unroll
-        for (int c = 0; c < 32; ++c) y += yp[c];
-      }
       T corr = T(0);
 #pragma unroll
       for (int k = 0; k < NB; ++k) corr += vr[k] * s_t[k] + wr[k] * s_t[NB + k];
