@@ -414,3 +414,39 @@ def test_qr_with_more_workgroups_in_a_launch_than_compute_units(device):
     assert torch.tril(r_lead, -1).abs().max().item() <= 1e-5 * r_lead.abs().max().item()
     residual = factor[:, :lead].double() @ torch.triu(r_lead) - matrix[:, :lead].double()
     assert residual.norm().item() <= 1e-5 * matrix[:, :lead].double().norm().item()
+
+
+def test_lost_messages_with_more_than_32_workgroups(device):
+    """n = 8704: 34 workgroups per panel launch, the size from which the Gram values travel in two
+    levels (shares summed by their owners, totals fetched by everybody).  With no patience for
+    another workgroup's message (spin limit 0) every wait of both levels must give up, leave the
+    kernel and poison Q, or, if every message happened to be there at the first poll, give a correct
+    Q; the next factorisation with the default limit is clean."""
+    from soap_tp_amd import _native
+    size = 8704
+    generator = torch.Generator(device=device).manual_seed(SEED + size)
+    matrix = torch.randn(size, size, device=device, generator=generator).T
+
+    def run():
+        factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+        ops.qr_2d_block_cyclic_(matrix.clone(), factor, size, BLOCK, GRID)
+        torch.cuda.synchronize()
+        return factor
+
+    def orthogonality(factor):
+        sample = factor[:, -384:].double()
+        return (sample.T @ sample - torch.eye(384, dtype=torch.float64, device=device)).abs().max().item()
+
+    assert not _native.device_error_flag(clear=True)
+    try:
+        _native.call("soapmi_set_option", b"message_spin_limit", 0)
+        factor = run()
+    finally:
+        _native.call("soapmi_set_option", b"message_spin_limit", 1 << 22)
+        reported = _native.device_error_flag(clear=True)
+    poisoned = bool(torch.isnan(factor).any())
+    assert poisoned or orthogonality(factor) <= 1e-5
+    assert reported == poisoned
+    factor = run()
+    assert torch.isfinite(factor).all() and orthogonality(factor) <= 1e-5
+    assert not _native.device_error_flag(clear=True)
