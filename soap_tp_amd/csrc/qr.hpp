@@ -668,7 +668,9 @@ __global__ __launch_bounds__(256) void qr_panel_persistent_kernel(float* __restr
 // Gram matrix, which a wavefront computes on the matrix cores: its 64 rows go through LDS once to
 // get from "lane = row" to the operand layout "lane = (row parity, column)", then 32
 // v_mfma_f32_32x32x2 instructions (operand a = operand b) accumulate X^T X.  The workgroups exchange
-// the upper triangle of that matrix (528 words) and the top block (1024 words) once, every
+// the upper triangle of that matrix (528 words) and the top block (1024 words) once (all-to-all up
+// to 32 workgroups; beyond that in two levels: a workgroup sums its share of the 528 values over
+// all workgroups, publishes the totals, and every workgroup fetches the totals), every
 // workgroup runs all Householder steps of the panel on [top block ; Gram] with the same guard as
 // above (a round ends before a column whose corrected norm has lost three quarters of its terms'
 // size, and that column opens a new round with a freshly computed Gram matrix), and then applies
