@@ -30,6 +30,7 @@ namespace soapmi {
 constexpr int kTrdNb = 32;        // panel width
 constexpr int kTrdTile = 128;     // tile edge of the matrix-vector product
 constexpr int kTrdMaxWg = 128;    // workgroups of the fused column kernel (256 rows each)
+constexpr int kTrdWideBelow = 256;  // tiles up to which the matrix-vector kernel runs 512 threads per tile (one tile per compute unit)
 
 template <typename T>
 struct TrdWorkspace {
@@ -384,14 +385,20 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
 // sums, slot s > b from tile (s, b)'s column sums, and slot b from the diagonal tile, which adds
 // both.  Every (slot, index) pair is written exactly once, so kernel D sums nb slots per index in a
 // fixed order and nothing has to be cleared.
-template <typename T>
-__global__ __launch_bounds__(256) void trd_symv_kernel(const T* __restrict__ A, int64_t lda, int n, int j,
-                                                       const T* __restrict__ v, T* __restrict__ y_part) {
+// QS = 1: 256 threads, a thread takes its row's 64 entries in two groups of 32 columns, one after
+// the other.  QS = 2: 512 threads, the two groups go to two sets of four wavefronts, so that a tile
+// is one trip to memory and one round of arithmetic instead of two each; the host picks it while
+// there are no more tiles than compute units (there the chain of one tile is the time of the launch;
+// a compute unit holds one such workgroup), and QS = 1, three tiles per compute unit, above.
+template <typename T, int QS>
+__global__ __launch_bounds__(256 * QS) void trd_symv_kernel(const T* __restrict__ A, int64_t lda, int n, int j,
+                                                            const T* __restrict__ v, T* __restrict__ y_part) {
   constexpr int TS = kTrdTile;
   __shared__ T s_v[TS];
-  __shared__ T s_direct[2][TS];
+  __shared__ T s_direct[2 * QS][TS];
   __shared__ T s_col[4][64];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+  const int q_first = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);  // 0 unless QS = 2
   // `half` is the same for all lanes of a wavefront: telling the compiler so moves the column
   // address arithmetic to the scalar unit
   const int row = tid & (TS - 1), half = __builtin_amdgcn_readfirstlane(tid >> 7);
@@ -412,16 +419,16 @@ __global__ __launch_bounds__(256) void trd_symv_kernel(const T* __restrict__ A, 
   const int rr = min(r, n - 1);
   const int limit = diagonal ? r : n - 1;  // last column that counts for this row
 #pragma unroll 1
-  for (int q = 0; q < 2; ++q) {  // 32 columns at a time
+  for (int q = q_first; q < 2; q += QS) {  // 32 columns at a time
     const int cq = c0 + 64 * half + 32 * q;
     T a[32];
 #pragma unroll
     for (int k = 0; k < 32; ++k) a[k] = A[rr + (int64_t)min(cq + k, n - 1) * lda];
-    if (q == 0) {
+    if (q == q_first) {
       // The tile's piece of v is requested behind the first 32 columns and published by a barrier
       // that waits for both: one trip to memory instead of two (from about 4 000 rows down a
       // compute unit has one tile or none, and the trips are the time).
-      if (tid < TS) s_v[tid] = (c0 + tid < n) ? v[c0 + tid] : T(0);
+      if (threadIdx.x < TS) s_v[threadIdx.x] = (c0 + (int)threadIdx.x < n) ? v[c0 + threadIdx.x] : T(0);
       vr = live ? v[r] : T(0);
       __syncthreads();
     }
@@ -436,13 +443,14 @@ __global__ __launch_bounds__(256) void trd_symv_kernel(const T* __restrict__ A, 
     const T total = wave_reduce_32<T>(cols, lane);
     if ((lane & 1) == 0) s_col[wave][32 * q + ((lane >> 1) & 31)] = total;
   }
-  s_direct[half][row] = acc0 + acc1;
+  s_direct[2 * q_first + half][row] = acc0 + acc1;
   __syncthreads();
-  if (tid < TS) {
-    // wavefronts 2*half and 2*half+1 hold the two row halves of column half `half`
+  if (threadIdx.x < TS) {
+    // wavefronts 2*half and 2*half+1 (of either set) hold the two row halves of column half `half`
     const int h = tid >> 6, k = tid & 63;
     const T column_sum = s_col[2 * h][k] + s_col[2 * h + 1][k];
-    const T row_sum = s_direct[0][tid] + s_direct[1][tid];
+    T row_sum = s_direct[0][tid] + s_direct[1][tid];
+    if constexpr (QS == 2) row_sum += s_direct[2][tid] + s_direct[3][tid];
     const int gr = o + rb * TS + tid, gc = c0 + tid;
     if (diagonal) {
       if (gr < n) y_part[(int64_t)rb * n + gr] = row_sum + column_sum;
@@ -489,8 +497,12 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
       const int i = j - p;
       const int nt = n - j - 1;
       const int nb = (int)ceil_div64(nt, kTrdTile);
-      hipLaunchKernelGGL((trd_symv_kernel<T>), dim3(nb * (nb + 1) / 2), dim3(256), 0, s, A, lda, n, j,
-                         ws.vc + (int64_t)i * ldw, ws.y_part);
+      if (nb * (nb + 1) / 2 <= kTrdWideBelow)
+        hipLaunchKernelGGL((trd_symv_kernel<T, 2>), dim3(nb * (nb + 1) / 2), dim3(512), 0, s, A, lda, n, j,
+                           ws.vc + (int64_t)i * ldw, ws.y_part);
+      else
+        hipLaunchKernelGGL((trd_symv_kernel<T, 1>), dim3(nb * (nb + 1) / 2), dim3(256), 0, s, A, lda, n, j,
+                           ws.vc + (int64_t)i * ldw, ws.y_part);
       grid = (int)ceil_div64(nt, 256);
       const int do_next = (j + 1 < pe) ? 1 : 0;
       hipLaunchKernelGGL((trd_column_kernel<T>), dim3(grid), dim3(256), 0, s, A, lda, n, p, j, 1, do_next, ws.vc, ws.vc2,
