@@ -1329,7 +1329,10 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
           static_for<t + 1, NB>([&](auto row) {
             constexpr int q = decltype(row)::value;
             // lower half: rounded exactly as the rows' owners do it further down, so that both hold
-            // the same numbers (u = 0 there; lane t itself has tc = 0)
+            // the same numbers (u = 0 there; lane t itself has tc = 0).  This matters: with the scale
+            // folded into tc once per step (one multiplication less per entry, results a rounding
+            // apart) the factorisation of a matrix with pairs of nearly equal columns lost its
+            // backward stability.
             x[q] = (x[q] - tc * (b[q] * h.scale)) - lane_value<q>(tc) * u;
           });
           size_diag += T(2) * fabsf(tc * w) + fabsf(tc * tc * s2gtt);
