@@ -1060,23 +1060,18 @@ __global__ __launch_bounds__(256) void qr_panel_gram_kernel(float* __restrict__ 
     load_own_row();
     lds_barrier();  // (not __syncthreads(): that would wait for the loads just issued)
     if (wave == 0) {
-      T w[NB], gcol[NB];
+      T w[NB];
 #pragma unroll
-      for (int i = 0; i < NB; ++i) {
-        w[i] = s_cw[lane & (NB - 1)][i];
-        gcol[i] = s_cg[i][lane & (NB - 1)];
-      }
+      for (int i = 0; i < NB; ++i) w[i] = s_cw[lane & (NB - 1)][i];
       static_for<0, NB>([&](auto step) {
         constexpr int i = decltype(step)::value;
         const T xi = lane_value<i>(tau_lane) * w[i];
         s_cx[i][lane & (NB - 1)] = -xi;  // (both halves of the wavefront hold the same 32 columns)
         static_for<i + 1, NB>([&](auto col) {
           constexpr int l = decltype(col)::value;
-          w[l] -= lane_value<l>(gcol[i]) * xi;
+          w[l] -= s_cg[i][l] * xi;  // (one address for all lanes: a broadcast read, four entries per instruction)
         });
-        // (the updates of a step stay in that step: left to itself the compiler gathers all updates
-        // of one w[l] into a chain in front of its use and reads the 496 entries of G ahead, through
-        // more scalar registers than there are)
+        // (the updates of a step stay in that step)
         static_for<i + 1, NB>([&](auto col) { keep_behind_wait(w[decltype(col)::value]); });
       });
     }
