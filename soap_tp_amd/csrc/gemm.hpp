@@ -371,7 +371,23 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
   if constexpr (PF > 1) {
     // Slab kt + 1 waits in register slot (kt + 1) % PF; once it has been stored to LDS the slot takes
     // the load of slab kt + 1 + PF.  The loop is unrolled by PF so that slots are compile-time indices.
-    for (int kt0 = 0; kt0 < nk; kt0 += PF) {
+    // While slab kt + 1 + PF exists an iteration has no tests in it: a load that is issued only
+    // under a condition makes the compiler wait for every load in flight before the next LDS store
+    // (it must assume the fewest younger loads), which empties the queue once per slab.
+    const int steady = max(0, nk - PF - 1) / PF * PF;
+    for (int kt0 = 0; kt0 < steady; kt0 += PF) {
+#pragma unroll
+      for (int u = 0; u < PF; ++u) {
+        const int buf = (kt0 + u) & 1, slot = (u + 1) % PF;
+        multiply_slab(buf);
+        store_slab<T, BM, BK, NT, Cfg::NVA, SA>(As[buf ^ 1], pa[slot], a_xc, tid);
+        store_slab<T, BN, BK, NT, Cfg::NVB, SB>(Bs[buf ^ 1], pb[slot], b_xc, tid);
+        fa.load(pa[slot]);
+        fb.load(pb[slot]);
+        __syncthreads();
+      }
+    }
+    for (int kt0 = steady; kt0 < nk; kt0 += PF) {
 #pragma unroll
       for (int u = 0; u < PF; ++u) {
         const int kt = kt0 + u;
