@@ -154,6 +154,47 @@ def test_rotate(shape, direction, device):
     assert abs(packed.norm().item() / matrix.norm().item() - 1) < 1e-5  # orthogonal invariance
 
 
+# ---- the product every MFMA stage runs on, through its own entry point ---------------------------
+# Closed form: C = alpha op(A) op(B) + beta C in fp64 on the CPU (what SLATE's gemm computes for the
+# reference's rotations, src/soap_tp/csrc/slate_bindings.cpp:257-273).  Shapes pick every path of the
+# kernel: the general path (odd sizes, padded leading dimensions), the 128 x 128 fast path, and the
+# 64 x 64 tile's fast path with K = 1 .. 9 slabs of 32 (its loop is peeled into a part that keeps two
+# slabs in flight and a tail; K = 32, 64, 96 have no steady part, 128 and 160 one pass of it, ...).
+PRODUCT_SHAPES = ((1, 1, 1), (3, 5, 7), (65, 33, 17), (130, 70, 200), (128, 128, 16), (256, 384, 64),
+                  (2048, 2048, 48), (2048, 2048, 256)) + tuple((64, 128, 32 * slabs) for slabs in range(1, 10)) + (
+                  (192, 64, 1024), (300, 129, 96))
+
+
+@pytest.mark.parametrize("shape", PRODUCT_SHAPES)
+@pytest.mark.parametrize("transposes", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_product_entry_point(shape, transposes, dtype, device):
+    from soap_tp_amd import _native
+
+    m, n, k = shape
+    trans_a, trans_b = transposes
+    if dtype == torch.float64 and m * n * k > 2048 * 2048 * 48:
+        pytest.skip("the fp64 product takes the same code path at the smaller size")
+    a = make_matrix(k if trans_a else m, m if trans_a else k, seed=SEED + m + 3 * k, dtype=dtype)
+    b = make_matrix(n if trans_b else k, k if trans_b else n, seed=SEED + n + 5 * k, dtype=dtype)
+    c = make_matrix(m, n, seed=SEED + m * n, dtype=dtype)
+    name = "soapmi_gemm_f32" if dtype == torch.float32 else "soapmi_gemm_f64"
+    tolerance = RTOL if dtype == torch.float32 else 1e-13
+    for alpha, beta, pad in ((1.0, 0.0, 0), (-0.5, 1.0, 0), (2.0, -0.25, 3)):
+        stored_a, stored_b = column_major(a, device, pad=pad), column_major(b, device, pad=2 * pad)
+        stored_c = column_major(c, device, pad=pad)
+        _native.call(name, trans_a, trans_b, m, n, k, alpha, stored_a.data_ptr(), stored_a.stride(1),
+                     stored_b.data_ptr(), stored_b.stride(1), beta, stored_c.data_ptr(), stored_c.stride(1),
+                     torch.cuda.current_stream().cuda_stream)
+        op_a = a.double().T if trans_a else a.double()
+        op_b = b.double().T if trans_b else b.double()
+        expected = alpha * (op_a @ op_b) + beta * c.double()
+        assert relative_l2(stored_c, expected) <= tolerance, (alpha, beta, pad)
+        if pad:  # nothing was written between the columns
+            between = torch.as_strided(stored_c, (pad, n), (1, m + pad), stored_c.storage_offset() + m)
+            assert torch.count_nonzero(between).item() == 0
+
+
 # ---- order, QR, power iteration (tests/unit/test_slate_bindings.py) ------------------------------
 @pytest.mark.parametrize("size", [8, 12, 9, 13, 100, 257])
 def test_estimated_order_qr_and_power_iteration(size, device):
