@@ -144,6 +144,31 @@ def test_eigh_f64_c_abi_directly(device):
         _native.call("soapmi_eigh_f64", a.data_ptr(), w.data_ptr(), q.data_ptr(), size, size - 1, size, None, 0, None)
 
 
+@pytest.mark.parametrize("size", [1, 2, 33, 200, 700])
+def test_eigh_f32_c_abi_directly(size, device):
+    """soapmi_eigh_f32 is the solver behind the `eigh` variant (torch.linalg.eigh on the float32
+    Gram matrix in the reference, src/soap_tp/ops/factorizations.py:446-469): ascending, input
+    destroyed, lower triangle referenced.  Against LAPACK in fp64 on the same float32 matrix."""
+    g = make_matrix(size, size + 5)
+    matrix = g @ g.T
+    a = column_major(torch.tril(matrix) + torch.triu(torch.full_like(matrix, 9.0), 1), device, pad=3)
+    q = column_major(torch.zeros(size, size), device, pad=1)
+    w = torch.zeros(size, dtype=torch.float32, device=device)
+    nbytes = _native.library().soapmi_eigh_workspace_bytes(size, 4)
+    work = torch.empty(max(1, nbytes), dtype=torch.uint8, device=device)
+    _native.call("soapmi_eigh_f32", a.data_ptr(), w.data_ptr(), q.data_ptr(), size, a.stride(1), q.stride(1),
+                 work.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+    exact = torch.tril(matrix).double()
+    exact = exact + torch.tril(exact, -1).T
+    expected = torch.linalg.eigvalsh(exact)
+    scale = expected.abs().max().item()
+    values, vectors = w.cpu().double(), q.cpu().double()
+    assert torch.all(values[1:] >= values[:-1])
+    assert (values - expected).abs().max().item() <= 1e-5 * scale
+    assert (vectors.T @ vectors - torch.eye(size, dtype=torch.float64)).abs().max().item() <= 1e-4
+    assert torch.linalg.matrix_norm(exact @ vectors - vectors * values).item() <= 5e-5 * torch.linalg.matrix_norm(exact).item()
+
+
 @pytest.mark.parametrize("kind", ["clusters", "glued_wilkinson", "block_diagonal"])
 def test_eigh_f64_with_heavy_deflation(kind, device):
     """Spectra that make the divide and conquer deflate: eigenvalues repeated in groups (rotations

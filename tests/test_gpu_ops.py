@@ -108,6 +108,35 @@ def test_permute_and_redistribute_are_exact(shape, device):
         ops.permute_2d_block_cyclic_(packed, shape, row_order, column_order[:-1], BLOCK, GRID)
 
 
+@pytest.mark.parametrize("shape", [(1, 1), (9, 13), (64, 96), (300, 129), (1000, 257), (4100, 36)])
+@pytest.mark.parametrize("orders", ["both", "rows", "columns", "neither"])
+def test_gather_entry_point_is_exact(shape, orders, device):
+    """soapmi_gather_f32, the out-of-place form of the permutation (out[i, j] = in[row_order[i],
+    col_order[j]], src/soap_tp/ops/optimizer.py:408); a NULL order is the identity.  Padded leading
+    dimensions on both sides; nothing may be written between the columns of the output."""
+    from soap_tp_amd import _native
+
+    rows, columns = shape
+    matrix = make_matrix(rows, columns, seed=SEED + rows)
+    generator = torch.Generator().manual_seed(SEED + columns)
+    row_order = torch.randperm(rows, generator=generator) if orders in ("both", "rows") else None
+    column_order = torch.randperm(columns, generator=generator) if orders in ("both", "columns") else None
+    source = column_major(matrix, device, pad=2)
+    target = column_major(torch.zeros(rows, columns), device, pad=5)
+    device_rows = row_order.to(device) if row_order is not None else None
+    device_columns = column_order.to(device) if column_order is not None else None
+    _native.call("soapmi_gather_f32", source.data_ptr(), source.stride(1), target.data_ptr(), target.stride(1), rows,
+                 columns, device_rows.data_ptr() if device_rows is not None else None,
+                 device_columns.data_ptr() if device_columns is not None else None,
+                 torch.cuda.current_stream().cuda_stream)
+    expected = oracle.permute(matrix, row_order if row_order is not None else torch.arange(rows),
+                              column_order if column_order is not None else torch.arange(columns))
+    assert torch.equal(target.cpu(), expected)
+    between = torch.as_strided(target, (5, columns), (1, rows + 5), target.storage_offset() + rows)
+    assert torch.count_nonzero(between).item() == 0
+    assert torch.equal(source.cpu(), matrix)  # the input is read only
+
+
 @pytest.mark.parametrize("shape", [(8, 12), (13, 9), (96, 160), (256, 384), (1024, 1024), (700, 1300), (2048, 512)])
 @pytest.mark.parametrize("row_major", [True, False])
 @pytest.mark.parametrize("mirror", [True, False])
