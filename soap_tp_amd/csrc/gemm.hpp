@@ -137,6 +137,7 @@ struct GemmTile {
   static_assert(KS == 1 || (KS - 1) * TM * TN * Mfma<T>::NACC * (NT / KS) <= 2 * BK * (BM + PAD + BN + PAD),
                 "the groups' accumulators are exchanged through the operands' LDS buffers");
   static_assert((BK * BM / VW) % NT == 0 && (BK * BN / VW) % NT == 0, "loader tiling");
+  static constexpr int LDS_ELEMS = 2 * BK * SA + 2 * BK * SB;  // two buffers of a K-slab of each operand
 };
 
 // Which 16-byte piece of a k-contiguous operand slab vector index v handles: KV pieces along k for
@@ -266,7 +267,8 @@ struct FastLoader {
 // MODE < 0: general path (any size, alignment and layout, tested at run time).
 // MODE in 0..3: fast path, bit 0 = A operand x-contiguous, bit 1 = B operand x-contiguous.
 template <typename T, class Cfg, class Epi, int MODE>
-__device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Epi& epi, const int wg, const int z) {
+__device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Epi& epi, const int wg, const int z,
+                                               T* __restrict__ smem) {
   using MF = Mfma<T>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
   constexpr int MI = Cfg::MI, KI = Cfg::KI, TM = Cfg::TM, TN = Cfg::TN;
@@ -274,7 +276,8 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
   constexpr bool FAST = MODE >= 0;
   constexpr bool AXC = (MODE & 1) != 0, BXC = (MODE & 2) != 0;
 
-  __shared__ __attribute__((aligned(16))) T smem[2 * BK * SA + 2 * BK * SB];
+  // (smem: Cfg::LDS_ELEMS elements of the kernel's LDS, 16-byte aligned.  Declared by the kernel, not
+  // here: a kernel that holds two instances of this body would otherwise get two arrays.)
   T(*As)[BK * SA] = reinterpret_cast<T(*)[BK * SA]>(smem);
   T(*Bs)[BK * SB] = reinterpret_cast<T(*)[BK * SB]>(smem + 2 * BK * SA);
 
@@ -472,7 +475,8 @@ __device__ __forceinline__ void gemm_tile_body(const GemmProblem<T>& p, const Ep
 
 template <typename T, class Cfg, class Epi, int MODE>
 __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi) {
-  gemm_tile_body<T, Cfg, Epi, MODE>(p, epi, blockIdx.x, blockIdx.y);
+  __shared__ __attribute__((aligned(16))) T smem[Cfg::LDS_ELEMS];
+  gemm_tile_body<T, Cfg, Epi, MODE>(p, epi, blockIdx.x, blockIdx.y, smem);
 }
 
 // Two independent products in one launch: workgroups [0, grid0) take the first problem, the rest
@@ -481,8 +485,9 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmProblem<T> p, Epi epi
 template <typename T, class Cfg, class Epi, int MODE0, int MODE1>
 __global__ __launch_bounds__(Cfg::NT) void gemm_pair_kernel(GemmProblem<T> p0, Epi e0, GemmProblem<T> p1, Epi e1,
                                                             int grid0) {
-  if ((int)blockIdx.x < grid0) gemm_tile_body<T, Cfg, Epi, MODE0>(p0, e0, blockIdx.x, 0);
-  else gemm_tile_body<T, Cfg, Epi, MODE1>(p1, e1, (int)blockIdx.x - grid0, 0);
+  __shared__ __attribute__((aligned(16))) T smem[Cfg::LDS_ELEMS];
+  if ((int)blockIdx.x < grid0) gemm_tile_body<T, Cfg, Epi, MODE0>(p0, e0, blockIdx.x, 0, smem);
+  else gemm_tile_body<T, Cfg, Epi, MODE1>(p1, e1, (int)blockIdx.x - grid0, 0, smem);
 }
 
 // One problem per blockIdx.z, described in device memory (sizes may be produced by earlier
@@ -496,7 +501,8 @@ template <typename T, class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void gemm_batched_kernel(const BatchedGemm<T>* __restrict__ batch) {
   const BatchedGemm<T> b = batch[blockIdx.z];
   if (b.p.M <= 0 || b.p.N <= 0) return;
-  gemm_tile_body<T, Cfg, EpiStore<T>, -1>(b.p, b.e, blockIdx.x, 0);
+  __shared__ __attribute__((aligned(16))) T smem[Cfg::LDS_ELEMS];
+  gemm_tile_body<T, Cfg, EpiStore<T>, -1>(b.p, b.e, blockIdx.x, 0, smem);
 }
 
 // The same product for blockIdx.z = 0 .. batch-1, with the operands and the result a fixed number of
@@ -507,7 +513,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_strided_kernel(GemmProblem<T> p,
   p.A += (int64_t)blockIdx.z * stride_a;
   p.B += (int64_t)blockIdx.z * stride_b;
   e.C += (int64_t)blockIdx.z * stride_c;
-  gemm_tile_body<T, Cfg, EpiStore<T>, -1>(p, e, blockIdx.x, 0);
+  __shared__ __attribute__((aligned(16))) T smem[Cfg::LDS_ELEMS];
+  gemm_tile_body<T, Cfg, EpiStore<T>, -1>(p, e, blockIdx.x, 0, smem);
 }
 
 // Device-side twin of make_problem for the default tile.
