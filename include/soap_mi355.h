@@ -63,6 +63,13 @@ const char* soapmi_last_error(void);
  *       panel's reflectors rides along in the launch of the next panel (extra workgroups update the
  *       columns behind that panel, the panel's own workgroups update their 32 columns themselves);
  *       with 0 it is a launch of its own between two panels.
+ *   "qr_super_block"  0, 256 or 1024 (default 0): the widest compact-WY reflector of the QR.  With
+ *       1024 the 256-column blocks are applied only inside a super-block of 1024 columns, and the
+ *       matrix beyond it (and the explicit Q) is updated once per super-block by products with
+ *       K = 1024; with 256 every block updates the whole trailing matrix (K = 256); 0 takes 1024 up
+ *       to n = 4096 and 256 above (the faster one on MI355X by 1 to 4 % either way).  1024 applies
+ *       where every panel runs on the whole-panel kernel ("qr_columns_per_round" 32, at most
+ *       "qr_persistent_max_workgroups" x 256 rows); other settings use 256.
  *   "persistent_workgroup_budget"  1..256 (default 256): the QR panel kernel and the
  *       tridiagonalisation's column kernel need all workgroups of a launch resident together (one per
  *       256 rows).  The library keeps count of the factorisations that may still be running on a

@@ -40,6 +40,8 @@ static std::atomic<int> g_qr_columns_per_round{kQrWholePanel};
 static std::atomic<int> g_refresh_streams{2};
 // 1 = a QR panel's in-block update rides along in the next panel's launch, 0 = a launch of its own
 static std::atomic<int> g_qr_carry_update{1};
+// widest compact-WY reflector of the QR: kQrSuper = three blocking levels, kBrMax = two, 0 = by size
+static std::atomic<int> g_qr_super_block{0};
 // tridiagonalisation of the eigensolver: kEighOneStage or kEighTwoStage (see soapmi_set_option)
 static std::atomic<int> g_eigh_algorithm{kEighOneStage};
 static std::mutex g_scratch_mutex;
@@ -354,6 +356,12 @@ int soapmi_set_option(const char* name, int64_t value) {
   if (strcmp(name, "qr_carry_update") == 0) {
     SOAPMI_REQUIRE(value == 0 || value == 1, "qr_carry_update must be 0 or 1");
     g_qr_carry_update.store((int)value);
+    return kOk;
+  }
+  if (strcmp(name, "qr_super_block") == 0) {
+    SOAPMI_REQUIRE(value == 0 || value == kBrMax || value == kQrSuper, "qr_super_block must be 0, %d or %d", kBrMax,
+                   kQrSuper);
+    g_qr_super_block.store((int)value);
     return kOk;
   }
   if (strcmp(name, "refresh_streams") == 0) {
@@ -779,7 +787,8 @@ int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t 
   if (rc) return rc;
   rc = qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws,
                                    g_qr_persistent_max_wg.load(), g_message_spin_limit.load(),
-                                   g_qr_columns_per_round.load(), report, g_qr_carry_update.load() != 0);
+                                   g_qr_columns_per_round.load(), report, g_qr_carry_update.load() != 0,
+                                   g_qr_super_block.load());
   const int rc_release = guard.release();
   return rc ? rc : rc_release;
 }

@@ -1681,39 +1681,45 @@ static inline void block_reflector_layout(WS& ws, int64_t n, BlockReflectorWs<T>
 // T12 = -T11 (G12 T22); all pairs of one span length are independent and share a launch, so a
 // 256-wide factor takes three levels (S = 32, 64, 128) of two products each.
 template <typename T>
-static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws, int nbw, const T* tau, T* Tm,
-                                    int first_block) {
+static inline int assemble_t_factor_ld(hipStream_t s, const T* gram, int ldg, T* mx, int ldmx, int nbw, const T* tau,
+                                       T* Tm, int ldt, int first_block) {
   using Small = typename SmallTile<T>::type;
   const int blocks = (int)ceil_div64(nbw, 32);
   if (first_block < blocks) {
     hipLaunchKernelGGL((larft32_kernel<T>), dim3(blocks - first_block), dim3(32 * larft_groups<T>()), 0, s,
-                       ws.gram + (int64_t)32 * first_block * (kBrMax + 1), kBrMax, 1, (int64_t)0, tau + 32 * first_block,
-                       nbw - 32 * first_block, Tm + (int64_t)32 * first_block * (kBrMax + 1), kBrMax);
+                       gram + (int64_t)32 * first_block * (ldg + 1), ldg, 1, (int64_t)0, tau + 32 * first_block,
+                       nbw - 32 * first_block, Tm + (int64_t)32 * first_block * (ldt + 1), ldt);
     SOAPMI_LAUNCH_CHECK();
   }
   for (int S = 32; S < nbw; S *= 2) {
-    const int64_t pair_stride = (int64_t)2 * S * (kBrMax + 1);  // from one pair's blocks to the next pair's
-    const int64_t off12 = (int64_t)S * kBrMax;                  // block (0, S) of a pair, relative to its block (0, 0)
-    const int64_t off22 = (int64_t)S * (kBrMax + 1);
-    const int full = nbw / (2 * S);                             // pairs whose right span is complete
-    const int right = nbw - (2 * S * full + S);                 // width of the last, shorter right span (<= 0: none)
-    int rc = gemm_strided_batch<T, Small>(s, S, S, S, T(1), ws.gram + off12, kBrMax, pair_stride, Tm + off22, kBrMax,
-                                          pair_stride, T(0), ws.mx + off12, kBrMax, pair_stride, full);
+    // from one pair's blocks to the next pair's; block (0, S) and (S, S) of a pair relative to its block (0, 0)
+    const int64_t pair_g = (int64_t)2 * S * (ldg + 1), pair_t = (int64_t)2 * S * (ldt + 1);
+    const int64_t pair_m = (int64_t)2 * S * (ldmx + 1);
+    const int64_t g12 = (int64_t)S * ldg, t12 = (int64_t)S * ldt, t22 = (int64_t)S * (ldt + 1), m12 = (int64_t)S * ldmx;
+    const int full = nbw / (2 * S);              // pairs whose right span is complete
+    const int right = nbw - (2 * S * full + S);  // width of the last, shorter right span (<= 0: none)
+    int rc = gemm_strided_batch<T, Small>(s, S, S, S, T(1), gram + g12, ldg, pair_g, Tm + t22, ldt, pair_t, T(0),
+                                          mx + m12, ldmx, pair_m, full);
     if (rc) return rc;
-    rc = gemm_strided_batch<T, Small>(s, S, S, S, T(-1), Tm, kBrMax, pair_stride, ws.mx + off12, kBrMax, pair_stride,
-                                      T(0), Tm + off12, kBrMax, pair_stride, full);
+    rc = gemm_strided_batch<T, Small>(s, S, S, S, T(-1), Tm, ldt, pair_t, mx + m12, ldmx, pair_m, T(0), Tm + t12, ldt,
+                                      pair_t, full);
     if (rc) return rc;
     if (right > 0) {
-      const int64_t base = (int64_t)full * pair_stride;
-      rc = gemm<T, Small>(s, 0, 0, S, right, right, T(1), ws.gram + base + off12, kBrMax, Tm + base + off22, kBrMax, T(0),
-                          ws.mx + base + off12, kBrMax);
+      rc = gemm<T, Small>(s, 0, 0, S, right, right, T(1), gram + full * pair_g + g12, ldg, Tm + full * pair_t + t22, ldt,
+                          T(0), mx + full * pair_m + m12, ldmx);
       if (rc) return rc;
-      rc = gemm<T, Small>(s, 0, 0, S, right, S, T(-1), Tm + base, kBrMax, ws.mx + base + off12, kBrMax, T(0),
-                          Tm + base + off12, kBrMax);
+      rc = gemm<T, Small>(s, 0, 0, S, right, S, T(-1), Tm + full * pair_t, ldt, mx + full * pair_m + m12, ldmx, T(0),
+                          Tm + full * pair_t + t12, ldt);
       if (rc) return rc;
     }
   }
   return kOk;
+}
+
+template <typename T>
+static inline int assemble_t_factor(hipStream_t s, const BlockReflectorWs<T>& ws, int nbw, const T* tau, T* Tm,
+                                    int first_block) {
+  return assemble_t_factor_ld<T>(s, ws.gram, kBrMax, ws.mx, kBrMax, nbw, tau, Tm, kBrMax, first_block);
 }
 
 // Number of K slices for a tall-skinny product with `tiles` output tiles, K = rows, an M x N
@@ -1925,6 +1931,24 @@ static inline void launch_extract_v(hipStream_t s, const T* A, int64_t lda, int 
                      dim3(256), 0, s, A, lda, rows, row0, col0, nbw, V, ldv, shift);
 }
 
+// State of the panel chain that runs through a whole factorisation.
+struct QrChainState {
+  unsigned seq_base = 0;       // sequence number of the next panel's first column (mailbox tags)
+  unsigned carried_total = 0;  // updating workgroups issued so far (what ws.sync[2] counts up to)
+};
+
+template <typename T>
+struct QrWorkspace;
+
+// The 32-column panels of the outer block [P, PE) of A (n x n): each panel is factored and applied
+// to the rest of the outer block.  Tm (ld kBrMax) receives diagonal 32-blocks of the outer factor
+// only on the launch-per-column path (*inner_done counts them).
+template <typename T>
+static inline int qr_outer_block_panels(hipStream_t s, T* A, int64_t lda, int n, int P, int PE, T* Tm,
+                                        const QrWorkspace<T>& ws, int persistent_max_wg, unsigned spin_limit,
+                                        int columns_per_round, bool carry_updates, QrChainState* chain,
+                                        int* inner_done, bool* v_written, bool* clean_in_a);
+
 // ---- QR driver -------------------------------------------------------------------------------
 // Mailbox words per workgroup and for the pivot rows: the larger of what the two persistent panel
 // kernels use (four columns per round: 4 x 32 and 4 x 32; whole panel: 9 x 64 and 32 x 32).
@@ -1934,6 +1958,7 @@ constexpr int kQrMailPivotWords = kQrNb * kQrNb;
 // for its batched loads, which read up to 31 rows past the last workgroup, used or not
 constexpr int kQrMailSpareWords = 48 * 64;
 constexpr int kQrWholePanel = kQrNb;  // columns_per_round value that selects qr_panel_gram_kernel
+constexpr int kQrSuper = 1024;        // widest super-block (third blocking level of the factorisation)
 
 template <typename T>
 struct QrWorkspace {
@@ -1945,6 +1970,13 @@ struct QrWorkspace {
   unsigned long long* mail_part;  // 2 x kQrPersistentMaxWg x kQrMailWords   mailboxes of the persistent panel kernels
   unsigned long long* mail_piv;   // 2 x kQrMailPivotWords
   unsigned* sync;  // [1] error flag of the persistent panel kernel, [2] count of finished updating workgroups
+  // third blocking level: super-blocks of up to kQrSuper columns (leading dimension sb_ld of all five)
+  int sb_ld;
+  T* t_super;  // super-blocks x sb_ld x sb_ld   compact-WY factors of the super-blocks
+  T* gram_s;   // sb_ld x sb_ld   row band k: V_k^T [V_0 .. V_k | C] of the super-block's k-th outer block
+  T* mx_s;     // sb_ld x sb_ld
+  T* w_s;      // sb_ld x n
+  T* w2_s;     // sb_ld x n
 };
 
 template <typename T, class WS>
@@ -1960,6 +1992,14 @@ static inline void qr_workspace_layout(WS& ws, int64_t n, QrWorkspace<T>* out) {
   q.mail_part = ws.template take<unsigned long long>((size_t)2 * kQrPersistentMaxWg * kQrMailWords + kQrMailSpareWords);
   q.mail_piv = ws.template take<unsigned long long>(2 * kQrMailPivotWords);
   q.sync = ws.template take<unsigned>(64);
+  // (padded: with a power of two as leading dimension the columns of T, W and W2 that a product
+  // reads together lie 4 KB apart and collide in the caches: measured 17 TFLOP/s for T^T W)
+  q.sb_ld = (int)std::min<int64_t>(kQrSuper, blocks * kBrMax) + 32;
+  q.t_super = ws.template take<T>((size_t)ceil_div64(n, kQrSuper) * q.sb_ld * q.sb_ld);
+  q.gram_s = ws.template take<T>((size_t)q.sb_ld * q.sb_ld);
+  q.mx_s = ws.template take<T>((size_t)q.sb_ld * q.sb_ld);
+  q.w_s = ws.template take<T>((size_t)q.sb_ld * n);
+  q.w2_s = ws.template take<T>((size_t)q.sb_ld * n);
   if (out) *out = q;
 }
 
@@ -1970,22 +2010,149 @@ static inline size_t qr_workspace_bytes(int64_t n) {
   return sizer.total();
 }
 
+template <typename T>
+static inline int qr_outer_block_panels(hipStream_t s, T* A, int64_t lda, int n, int P, int PE, T* Tm,
+                                        const QrWorkspace<T>& ws, int persistent_max_wg, unsigned spin_limit,
+                                        int columns_per_round, bool carry_updates, QrChainState* chain,
+                                        int* inner_done, bool* v_written, bool* clean_in_a) {
+  const int NB = kQrNb, OB = kBrMax;
+  const int64_t ldv = n;
+  int rc;
+  int pending_p = -1, pending_nwg = 0, pending_buffer = 0;  // a panel whose in-block update has not been issued
+  for (int p = P; p < PE; p += NB) {
+    const int pe = std::min(PE, p + NB), nbw = pe - p;
+    const int rows = n - p;
+    const int nwg = (int)ceil_div64(rows, 256);
+    T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
+    T* piv[2] = {ws.piv, ws.piv + NB};
+    // this panel's reflectors inside the outer block's n x 128 buffer (origin: row P, column P)
+    BlockReflectorWs<T> inner = ws.br;
+    inner.v = ws.br.v + (p - P) + (int64_t)(p - P) * ldv;
+    bool slices_by_panel = false;
+    if (nwg <= persistent_max_wg && columns_per_round == kQrWholePanel) {
+      // (a full panel with columns of the outer block behind it also leaves its slices of V^T [V | C];
+      // two slice buffers alternate, since a launch may read the earlier panel's while writing its own)
+      slices_by_panel = pe < PE && nbw == NB;
+      T* slice_buffer[2] = {ws.br.splitk, ws.br.splitk + (size_t)kBrSplits * kBrMax * ldv / 2};
+      PanelCarry carry{};
+      if (pending_p >= 0 && nbw == NB) {
+        // the earlier panel's in-block update rides along in this launch
+        const int groups = (int)ceil_div64(PE - pe, kPanelApplyCols);
+        carry.slices = slice_buffer[pending_buffer];
+        carry.splits = pending_nwg;
+        carry.slab = (int64_t)NB * (PE - pending_p);
+        carry.nc = PE - p;
+        carry.tau = ws.tau + pending_p;
+        carry.v = ws.br.v + (p - P) + (int64_t)(pending_p - P) * ldv;
+        carry.apply_row_blocks = nwg;
+        carry.apply_wgs = nwg * groups;
+        carry.done_counter = ws.sync + 2;
+        chain->carried_total += (unsigned)carry.apply_wgs;
+        carry.done_target = chain->carried_total;
+        pending_p = -1;
+      } else if (pending_p >= 0) {
+        // (a last, narrower panel: the earlier panel's update as a launch of its own)
+        hipLaunchKernelGGL(panel_apply_kernel,
+                           dim3((unsigned)ceil_div64(n - pending_p, 256), (unsigned)ceil_div64(PE - p, kPanelApplyCols)),
+                           dim3(256), 0, s, slice_buffer[pending_buffer], pending_nwg, (int64_t)NB * (PE - pending_p),
+                           PE - p, ws.tau + pending_p, ws.br.v + (pending_p - P) + (int64_t)(pending_p - P) * ldv, ldv,
+                           A + pending_p + (int64_t)p * lda, lda, n - pending_p);
+        SOAPMI_LAUNCH_CHECK();
+        pending_p = -1;
+      }
+      const int out_buffer = pending_buffer ^ 1;
+      hipLaunchKernelGGL(qr_panel_gram_kernel, dim3(nwg + carry.apply_wgs), dim3(256), 0, s, A, lda, n, p, pe,
+                         ws.mail_part, ws.mail_piv, ws.tau, chain->seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
+                         ws.br.v + (int64_t)(p - P) * ldv, ldv, P, slices_by_panel ? slice_buffer[out_buffer] : nullptr,
+                         PE - pe, (int64_t)NB * (PE - p), carry);
+      chain->seq_base += (unsigned)nbw;
+      if (slices_by_panel) {
+        pending_buffer = out_buffer;
+        if (carry_updates) {
+          pending_p = p;
+          pending_nwg = nwg;
+        } else {
+          hipLaunchKernelGGL(panel_apply_kernel,
+                             dim3((unsigned)nwg, (unsigned)ceil_div64(PE - pe, kPanelApplyCols)), dim3(256), 0, s,
+                             slice_buffer[out_buffer], nwg, (int64_t)NB * (PE - p), PE - pe, ws.tau + p, inner.v, ldv,
+                             A + p + (int64_t)pe * lda, lda, rows);
+        }
+      }
+    } else if (nwg <= persistent_max_wg) {
+      *clean_in_a = false;
+      hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
+                         ws.mail_piv, ws.tau, chain->seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
+                         ws.br.v + (int64_t)(p - P) * ldv, ldv, P, columns_per_round);
+      chain->seq_base += (unsigned)nbw;
+    } else {
+      for (int j = p - 1; j < pe; ++j) {
+        const int in = (j - p + 1) & 1, out = in ^ 1;
+        hipLaunchKernelGGL((qr_panel_step_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, j, part[in],
+                           piv[in], part[out], piv[out], ws.tau, nwg);
+      }
+      *v_written = false;
+      *clean_in_a = false;
+    }
+    SOAPMI_LAUNCH_CHECK();
+    if (slices_by_panel) {
+      // (the in-block update is on its way or rides along with the next panel)
+    } else if (pe < PE && *v_written) {
+      // The panel's reflectors act on the rest of the outer block only.  One product gives the
+      // slices of V^T [V | C] (the panel's own columns of A hold V in clean form); the middle
+      // factor T^T is applied as a triangular solve with V^T V, so no T is needed here: the
+      // diagonal blocks of the outer factor are all built after the block's last panel.
+      using Skinny = typename SkinnyTile<T>::type;
+      const int ncols = PE - p, nc = PE - pe;
+      int slices = 1;
+      rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, ncols, rows, inner.v, ldv, A + p + (int64_t)p * lda, lda,
+                                       split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
+                                       ws.br.splitk, &slices);
+      if (rc) return rc;
+      if (nbw == NB) {
+        hipLaunchKernelGGL(panel_apply_kernel, dim3((unsigned)ceil_div64(rows, 256), (unsigned)ceil_div64(nc, kPanelApplyCols)),
+                           dim3(256), 0, s, ws.br.splitk, slices, (int64_t)nbw * ncols, nc, ws.tau + p, inner.v, ldv,
+                           A + p + (int64_t)pe * lda, lda, rows);
+        SOAPMI_LAUNCH_CHECK();
+      } else {
+        hipLaunchKernelGGL((reflector_w2_solve_kernel<T>), dim3((unsigned)ceil_div64(nc, kW2SolveCols)), dim3(256), 0, s,
+                           ws.br.splitk, slices, (int64_t)nbw * ncols, nbw, nc, ws.tau + p, ws.br.w2, kBrMax);
+        SOAPMI_LAUNCH_CHECK();
+        rc = gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), inner.v, ldv, ws.br.w2, kBrMax, T(1), A + p + (int64_t)pe * lda, lda);
+        if (rc) return rc;
+      }
+    } else if (pe < PE) {
+      T* Tin = Tm + (int64_t)(p - P) * (OB + 1);  // diagonal block of the outer factor
+      launch_extract_v<T>(s, A, lda, rows, p, p, nbw, inner.v, ldv);
+      int slices = 1;  // V^T V stays in split-K slices; the factor kernel sums them while loading
+      rc = gemm_to_partials<T, typename SkinnyTile<T>::type>(s, 1, 0, nbw, nbw, rows, inner.v, ldv, inner.v, ldv,
+                                                             split_count(1, rows, nbw, nbw, ldv), inner.splitk,
+                                                             &slices);
+      if (rc) return rc;
+      hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(32 * larft_groups<T>()), 0, s, inner.splitk, nbw, slices,
+                         (int64_t)nbw * nbw, ws.tau + p, nbw, Tin, OB);
+      SOAPMI_LAUNCH_CHECK();
+      rc = apply_block_reflector<T>(s, inner, Tin, true, rows, nbw, PE - pe, ldv, A + p + (int64_t)pe * lda, lda);
+      if (rc) return rc;
+      ++*inner_done;
+    }
+  }
+  return kOk;
+}
+
 // geqrf in place on A (n x n), then the explicit Q into Qout (n x n).  A is destroyed.
 // Two levels of blocking: 32-column panels (register-resident column steps) are applied only
 // inside their kBrMax-column outer block; the trailing matrix and Q see kBrMax-wide block
 // reflectors, whose products have K = kBrMax and run on the full-size MFMA tile.
 template <typename T>
-static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
-                                       const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
-                                       unsigned spin_limit = kQrSpinLimit, int columns_per_round = kQrRoundMax,
-                                       int* report = nullptr, bool carry_updates = true) {
+static inline int qr_factor_and_form_q_two_level(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
+                                                 const QrWorkspace<T>& ws, int persistent_max_wg, unsigned spin_limit,
+                                                 int columns_per_round, int* report, bool carry_updates) {
   const int NB = kQrNb, OB = kBrMax;
   const int blocks = (int)ceil_div64(n, OB);
   const int64_t ldv = n;
   int rc;
   static_assert(std::is_same<T, float>::value, "the persistent panel kernel packs float values into its mailboxes");
-  unsigned seq_base = 0;
-  unsigned carried_total = 0;  // updating workgroups issued so far (what ws.sync[2] counts up to)
+  QrChainState chain;
   std::vector<char> block_clean((size_t)blocks, 0);  // outer blocks whose columns of A hold V in clean form
   hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
   {
@@ -2002,126 +2169,11 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
     const int P = bi * OB, PE = std::min(n, P + OB), obw = PE - P;
     T* Tm = ws.t_all + (size_t)bi * OB * OB;
     int inner_done = 0;
-    bool v_written = true;  // the panel kernels leave the block's reflectors in ws.br.v
-    int pending_p = -1, pending_nwg = 0, pending_buffer = 0;  // a panel whose in-block update has not been issued
-    bool clean_in_a = true;  // every panel so far left V in clean form in A too (the whole-panel kernel does)
-    for (int p = P; p < PE; p += NB) {
-      const int pe = std::min(PE, p + NB), nbw = pe - p;
-      const int rows = n - p;
-      const int nwg = (int)ceil_div64(rows, 256);
-      T* part[2] = {ws.part, ws.part + (size_t)nwg * NB};
-      T* piv[2] = {ws.piv, ws.piv + NB};
-      // this panel's reflectors inside the outer block's n x 128 buffer (origin: row P, column P)
-      BlockReflectorWs<T> inner = ws.br;
-      inner.v = ws.br.v + (p - P) + (int64_t)(p - P) * ldv;
-      bool slices_by_panel = false;
-      if (nwg <= persistent_max_wg && columns_per_round == kQrWholePanel) {
-        // (a full panel with columns of the outer block behind it also leaves its slices of V^T [V | C];
-        // two slice buffers alternate, since a launch may read the earlier panel's while writing its own)
-        slices_by_panel = pe < PE && nbw == NB;
-        T* slice_buffer[2] = {ws.br.splitk, ws.br.splitk + (size_t)kBrSplits * kBrMax * ldv / 2};
-        PanelCarry carry{};
-        if (pending_p >= 0 && nbw == NB) {
-          // the earlier panel's in-block update rides along in this launch
-          const int groups = (int)ceil_div64(PE - pe, kPanelApplyCols);
-          carry.slices = slice_buffer[pending_buffer];
-          carry.splits = pending_nwg;
-          carry.slab = (int64_t)NB * (PE - pending_p);
-          carry.nc = PE - p;
-          carry.tau = ws.tau + pending_p;
-          carry.v = ws.br.v + (p - P) + (int64_t)(pending_p - P) * ldv;
-          carry.apply_row_blocks = nwg;
-          carry.apply_wgs = nwg * groups;
-          carry.done_counter = ws.sync + 2;
-          carried_total += (unsigned)carry.apply_wgs;
-          carry.done_target = carried_total;
-          pending_p = -1;
-        } else if (pending_p >= 0) {
-          // (a last, narrower panel: the earlier panel's update as a launch of its own)
-          hipLaunchKernelGGL(panel_apply_kernel,
-                             dim3((unsigned)ceil_div64(n - pending_p, 256), (unsigned)ceil_div64(PE - p, kPanelApplyCols)),
-                             dim3(256), 0, s, slice_buffer[pending_buffer], pending_nwg, (int64_t)NB * (PE - pending_p),
-                             PE - p, ws.tau + pending_p, ws.br.v + (pending_p - P) + (int64_t)(pending_p - P) * ldv, ldv,
-                             A + pending_p + (int64_t)p * lda, lda, n - pending_p);
-          SOAPMI_LAUNCH_CHECK();
-          pending_p = -1;
-        }
-        const int out_buffer = pending_buffer ^ 1;
-        hipLaunchKernelGGL(qr_panel_gram_kernel, dim3(nwg + carry.apply_wgs), dim3(256), 0, s, A, lda, n, p, pe,
-                           ws.mail_part, ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
-                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, slices_by_panel ? slice_buffer[out_buffer] : nullptr,
-                           PE - pe, (int64_t)NB * (PE - p), carry);
-        seq_base += (unsigned)nbw;
-        if (slices_by_panel) {
-          pending_buffer = out_buffer;
-          if (carry_updates) {
-            pending_p = p;
-            pending_nwg = nwg;
-          } else {
-            hipLaunchKernelGGL(panel_apply_kernel,
-                               dim3((unsigned)nwg, (unsigned)ceil_div64(PE - pe, kPanelApplyCols)), dim3(256), 0, s,
-                               slice_buffer[out_buffer], nwg, (int64_t)NB * (PE - p), PE - pe, ws.tau + p, inner.v, ldv,
-                               A + p + (int64_t)pe * lda, lda, rows);
-          }
-        }
-      } else if (nwg <= persistent_max_wg) {
-        clean_in_a = false;
-        hipLaunchKernelGGL(qr_panel_persistent_kernel, dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, ws.mail_part,
-                           ws.mail_piv, ws.tau, seq_base, reinterpret_cast<int*>(ws.sync + 1), nwg, spin_limit,
-                           ws.br.v + (int64_t)(p - P) * ldv, ldv, P, columns_per_round);
-        seq_base += (unsigned)nbw;
-      } else {
-        for (int j = p - 1; j < pe; ++j) {
-          const int in = (j - p + 1) & 1, out = in ^ 1;
-          hipLaunchKernelGGL((qr_panel_step_kernel<T>), dim3(nwg), dim3(256), 0, s, A, lda, n, p, pe, j, part[in],
-                             piv[in], part[out], piv[out], ws.tau, nwg);
-        }
-        v_written = false;
-        clean_in_a = false;
-      }
-      SOAPMI_LAUNCH_CHECK();
-      if (slices_by_panel) {
-        // (the in-block update is on its way or rides along with the next panel)
-      } else if (pe < PE && v_written) {
-        // The panel's reflectors act on the rest of the outer block only.  One product gives the
-        // slices of V^T [V | C] (the panel's own columns of A hold V in clean form); the middle
-        // factor T^T is applied as a triangular solve with V^T V, so no T is needed here: the
-        // diagonal blocks of the outer factor are all built after the block's last panel.
-        using Skinny = typename SkinnyTile<T>::type;
-        const int ncols = PE - p, nc = PE - pe;
-        int slices = 1;
-        rc = gemm_to_partials<T, Skinny>(s, 1, 0, nbw, ncols, rows, inner.v, ldv, A + p + (int64_t)p * lda, lda,
-                                         split_count(ceil_div64(ncols, Skinny::BN), rows, nbw, ncols, ldv),
-                                         ws.br.splitk, &slices);
-        if (rc) return rc;
-        if (nbw == NB) {
-          hipLaunchKernelGGL(panel_apply_kernel, dim3((unsigned)ceil_div64(rows, 256), (unsigned)ceil_div64(nc, kPanelApplyCols)),
-                             dim3(256), 0, s, ws.br.splitk, slices, (int64_t)nbw * ncols, nc, ws.tau + p, inner.v, ldv,
-                             A + p + (int64_t)pe * lda, lda, rows);
-          SOAPMI_LAUNCH_CHECK();
-        } else {
-          hipLaunchKernelGGL((reflector_w2_solve_kernel<T>), dim3((unsigned)ceil_div64(nc, kW2SolveCols)), dim3(256), 0, s,
-                             ws.br.splitk, slices, (int64_t)nbw * ncols, nbw, nc, ws.tau + p, ws.br.w2, kBrMax);
-          SOAPMI_LAUNCH_CHECK();
-          rc = gemm<T>(s, 0, 0, rows, nc, nbw, T(-1), inner.v, ldv, ws.br.w2, kBrMax, T(1), A + p + (int64_t)pe * lda, lda);
-          if (rc) return rc;
-        }
-      } else if (pe < PE) {
-        T* Tin = Tm + (int64_t)(p - P) * (OB + 1);  // diagonal block of the outer factor
-        launch_extract_v<T>(s, A, lda, rows, p, p, nbw, inner.v, ldv);
-        int slices = 1;  // V^T V stays in split-K slices; the factor kernel sums them while loading
-        rc = gemm_to_partials<T, typename SkinnyTile<T>::type>(s, 1, 0, nbw, nbw, rows, inner.v, ldv, inner.v, ldv,
-                                                               split_count(1, rows, nbw, nbw, ldv), inner.splitk,
-                                                               &slices);
-        if (rc) return rc;
-        hipLaunchKernelGGL((larft32_kernel<T>), dim3(1), dim3(32 * larft_groups<T>()), 0, s, inner.splitk, nbw, slices,
-                           (int64_t)nbw * nbw, ws.tau + p, nbw, Tin, OB);
-        SOAPMI_LAUNCH_CHECK();
-        rc = apply_block_reflector<T>(s, inner, Tin, true, rows, nbw, PE - pe, ldv, A + p + (int64_t)pe * lda, lda);
-        if (rc) return rc;
-        ++inner_done;
-      }
-    }
+    bool v_written = true;   // the panel kernels leave the block's reflectors in ws.br.v
+    bool clean_in_a = true;  // every panel left V in clean form in A too (the whole-panel kernel does)
+    rc = qr_outer_block_panels<T>(s, A, lda, n, P, PE, Tm, ws, persistent_max_wg, spin_limit, columns_per_round,
+                                  carry_updates, &chain, &inner_done, &v_written, &clean_in_a);
+    if (rc) return rc;
     const int rows = n - P;
     if (!v_written) launch_extract_v<T>(s, A, lda, rows, P, P, obw, ws.br.v, ldv);
     block_clean[bi] = clean_in_a ? 1 : 0;
@@ -2172,6 +2224,180 @@ static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout
                      reinterpret_cast<const int*>(ws.sync + 1), report);
   SOAPMI_LAUNCH_CHECK();
   return kOk;
+}
+
+// Zeroes, in the columns of the super-block [S0, S1) of A, the rows of the super-block above each
+// outer block's own rows (entries of R that no one reads), so that the super-block's columns hold
+// its reflectors in clean form from row S0 on.  Grid: (row chunks of 256, outer blocks 1 ..).
+template <typename T>
+__global__ __launch_bounds__(256) void zero_above_blocks_kernel(T* __restrict__ A, int64_t lda, int S0, int S1) {
+  const int P = S0 + kBrMax * ((int)blockIdx.y + 1), PE = min(S1, P + kBrMax);
+  const int r = S0 + (int)blockIdx.x * 256 + (int)threadIdx.x;
+  if (r >= P) return;
+  for (int c = P; c < PE; ++c) A[r + (int64_t)c * lda] = T(0);
+}
+
+// Slice count of a product with a long K whose partial results go to the block-reflector split-K
+// buffer (`capacity` elements).
+static inline int split_count_capacity(int64_t tiles, int rows, int M, int N, int64_t capacity) {
+  // split_count sizes by kBrSplits * kBrMax * ldv: hand it the ldv that gives `capacity`
+  return split_count(tiles, rows, M, N, capacity / ((int64_t)kBrSplits * kBrMax));
+}
+
+// C (rows x nc, ld ldc) <- (I - V op(T) V^T) C for a reflector block of any width k (V rows x k in
+// clean form; T k x k upper triangular, ld ldt); W and W2 (k x nc, ld ldw) are scratch.
+template <typename T>
+static inline int apply_wide_reflector(hipStream_t s, const T* V, int64_t ldv, const T* Tm, int ldt, bool transT,
+                                       int rows, int k, int nc, T* C, int64_t ldc, T* W, T* W2, int ldw, T* splitk,
+                                       int64_t splitk_capacity) {
+  using Wide = typename DefaultTile<T>::type;
+  if (nc <= 0 || rows <= 0 || k <= 0) return kOk;
+  const int64_t tiles = ceil_div64(nc, Wide::BN) * ceil_div64(k, Wide::BM);
+  const int splits = split_count_capacity(tiles, rows, k, nc, splitk_capacity);
+  int rc = gemm<T>(s, 1, 0, k, nc, rows, T(1), V, ldv, C, ldc, T(0), W, ldw, splits, splitk);
+  if (rc) return rc;
+  rc = gemm<T>(s, transT ? 1 : 0, 0, k, nc, k, T(1), Tm, ldt, W, ldw, T(0), W2, ldw);
+  if (rc) return rc;
+  return gemm<T>(s, 0, 0, rows, nc, k, T(-1), V, ldv, W2, ldw, T(1), C, ldc);
+}
+
+// Three levels of blocking: panels of 32 columns inside outer blocks of kBrMax columns as above, and
+// outer blocks inside super-blocks of kQrSuper columns.  An outer block's reflectors are applied only
+// to the rest of its super-block; everything beyond sees the super-block as one kQrSuper-wide
+// compact-WY reflector, so the bulk of the trailing updates and of the Q formation are products
+// with K = kQrSuper, which re-read and re-write the trailing matrix a quarter as often as K = kBrMax
+// ones.  The super-block's factor T has the outer blocks' factors on its diagonal and above it
+// T12 = -T11 (V1^T V2) T22 by doubling (spans of 256, 512); the cross products V_k^T V_l (l < k) come
+// out of the product that an outer block needs anyway, V_k^T A[:, super-block]: its columns left of
+// the block are the earlier blocks' reflectors, the block's own columns give V_k^T V_k and the rest
+// V_k^T C.  Requires every panel to run on the whole-panel kernel (which leaves V in clean form in A).
+template <typename T>
+static inline int qr_factor_and_form_q_three_level(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
+                                                   const QrWorkspace<T>& ws, int persistent_max_wg,
+                                                   unsigned spin_limit, int* report, bool carry_updates) {
+  using Wide = typename DefaultTile<T>::type;
+  const int OB = kBrMax, SB = kQrSuper, LD = ws.sb_ld;
+  const int supers = (int)ceil_div64(n, SB);
+  const int64_t ldv = n;
+  const int64_t splitk_capacity = (int64_t)kBrSplits * kBrMax * n;
+  int rc;
+  QrChainState chain;
+  hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3(1), dim3(64), 0, s, ws.sync, 64);
+  {
+    const int words = (int)(reinterpret_cast<unsigned*>(ws.mail_piv + 2 * kQrMailPivotWords) -
+                            reinterpret_cast<unsigned*>(ws.mail_part));
+    hipLaunchKernelGGL((fill_zero_kernel<unsigned>), dim3((words + 255) / 256), dim3(256), 0, s,
+                       reinterpret_cast<unsigned*>(ws.mail_part), words);
+  }
+  {
+    const int64_t count = (int64_t)supers * LD * LD;
+    hipLaunchKernelGGL((fill_zero_kernel<T>), dim3((unsigned)ceil_div64(count, 256)), dim3(256), 0, s, ws.t_super,
+                       (int)count);
+  }
+  SOAPMI_LAUNCH_CHECK();
+  // ---- factorisation ----
+  for (int si = 0; si < supers; ++si) {
+    const int S0 = si * SB, S1 = std::min(n, S0 + SB), sbw = S1 - S0;
+    T* Ts = ws.t_super + (size_t)si * LD * LD;
+    for (int P = S0; P < S1; P += OB) {
+      const int PE = std::min(S1, P + OB), obw = PE - P, rows = n - P;
+      T* Tm = Ts + (int64_t)(P - S0) * (LD + 1);  // diagonal block of the super-block's factor
+      int inner_done = 0;
+      bool v_written = true, clean_in_a = true;
+      rc = qr_outer_block_panels<T>(s, A, lda, n, P, PE, (T*)nullptr, ws, persistent_max_wg, spin_limit, kQrWholePanel,
+                                    carry_updates, &chain, &inner_done, &v_written, &clean_in_a);
+      if (rc) return rc;
+      if (!v_written || !clean_in_a || inner_done != 0) {
+        set_error("internal error: a QR panel left the whole-panel path");
+        return kRuntimeError;
+      }
+      // row band of the super-block's Gram matrix: V_k^T A[P:, S0:S1]
+      T* band = ws.gram_s + (P - S0);
+      const int64_t tiles = ceil_div64(sbw, Wide::BN) * ceil_div64(obw, Wide::BM);
+      rc = gemm<T>(s, 1, 0, obw, sbw, rows, T(1), ws.br.v, ldv, A + P + (int64_t)S0 * lda, lda, T(0), band, LD,
+                   split_count_capacity(tiles, rows, obw, sbw, splitk_capacity), ws.br.splitk);
+      if (rc) return rc;
+      rc = assemble_t_factor_ld<T>(s, band + (int64_t)(P - S0) * LD, LD, ws.br.mx, kBrMax, obw, ws.tau + P, Tm, LD, 0);
+      if (rc) return rc;
+      const int nc = S1 - PE;
+      if (nc > 0) {  // the rest of the super-block: C <- C - V_k T_k^T (V_k^T C)
+        rc = gemm<T>(s, 1, 0, obw, nc, obw, T(1), Tm, LD, band + (int64_t)(PE - S0) * LD, LD, T(0), ws.br.w2, kBrMax);
+        if (rc) return rc;
+        rc = gemm<T>(s, 0, 0, rows, nc, obw, T(-1), ws.br.v, ldv, ws.br.w2, kBrMax, T(1), A + P + (int64_t)PE * lda, lda);
+        if (rc) return rc;
+      }
+    }
+    // blocks of T above the diagonal blocks, by doubling: spans of kBrMax, 2 kBrMax, ...
+    for (int S = OB; S < sbw; S *= 2) {
+      for (int o = 0; o + S < sbw; o += 2 * S) {
+        const int r = std::min(S, sbw - (o + S));  // width of the right span
+        const T* g21 = ws.gram_s + (o + S) + (int64_t)o * LD;       // V2^T V1 (r x S)
+        const T* t11 = Ts + (int64_t)o * (LD + 1);
+        const T* t22 = Ts + (int64_t)(o + S) * (LD + 1);
+        T* t12 = Ts + o + (int64_t)(o + S) * LD;
+        rc = gemm<T>(s, 1, 0, S, r, r, T(1), g21, LD, t22, LD, T(0), ws.mx_s, LD);
+        if (rc) return rc;
+        rc = gemm<T>(s, 0, 0, S, r, S, T(-1), t11, LD, ws.mx_s, LD, T(0), t12, LD);
+        if (rc) return rc;
+      }
+    }
+    if (sbw > OB) {
+      hipLaunchKernelGGL((zero_above_blocks_kernel<T>), dim3((unsigned)ceil_div64(sbw - OB, 256), (unsigned)ceil_div64(sbw - OB, OB)),
+                         dim3(256), 0, s, A, lda, S0, S1);
+      SOAPMI_LAUNCH_CHECK();
+    }
+    // everything beyond the super-block: C <- H^T C = C - V T^T V^T C with K = sbw
+    rc = apply_wide_reflector<T>(s, A + S0 + (int64_t)S0 * lda, lda, Ts, LD, true, n - S0, sbw, n - S1,
+                                 A + S0 + (int64_t)S1 * lda, lda, ws.w_s, ws.w2_s, LD, ws.br.splitk, splitk_capacity);
+    if (rc) return rc;
+  }
+  // ---- explicit Q, super-blocks in reverse ----
+  for (int si = supers - 1; si >= 0; --si) {
+    const int S0 = si * SB, S1 = std::min(n, S0 + SB), sbw = S1 - S0;
+    const T* Ts = ws.t_super + (size_t)si * LD * LD;
+    // columns beyond the super-block already hold Q of the later ones: C <- (I - V T V^T) C
+    rc = apply_wide_reflector<T>(s, A + S0 + (int64_t)S0 * lda, lda, Ts, LD, false, n - S0, sbw, n - S1,
+                                 Qout + S0 + (int64_t)S1 * ldq, ldq, ws.w_s, ws.w2_s, LD, ws.br.splitk, splitk_capacity);
+    if (rc) return rc;
+    // own columns, all outer blocks at once: [I;0] - V (T V1^T).  (Block by block, each applied to the
+    // later columns of the super-block, would be half the arithmetic, in products of a few tiles each
+    // that run at a quarter of the rate.)
+    const T* V = A + S0 + (int64_t)S0 * lda;
+    rc = gemm<T>(s, 0, 1, sbw, sbw, sbw, T(1), Ts, LD, V, lda, T(0), ws.mx_s, LD);
+    if (rc) return rc;
+    rc = gemm<T>(s, 0, 0, n - S0, sbw, sbw, T(-1), V, lda, ws.mx_s, LD, T(0), Qout + S0 + (int64_t)S0 * ldq, ldq);
+    if (rc) return rc;
+    hipLaunchKernelGGL((orgqr_panel_fix_kernel<T>), dim3((unsigned)ceil_div64(S1, 256)), dim3(256), 0, s, Qout, ldq, S0,
+                       sbw);
+    SOAPMI_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL((poison_on_error_kernel<T>), dim3(1), dim3(64), 0, s, Qout, ldq, n,
+                     reinterpret_cast<const int*>(ws.sync + 1), report);
+  SOAPMI_LAUNCH_CHECK();
+  return kOk;
+}
+
+// geqrf in place on A (n x n), then the explicit Q into Qout (n x n).  A is destroyed.  `super_block`:
+// kQrSuper selects the three-level blocking where every panel can run on the whole-panel kernel,
+// kBrMax (and every other panel setting) the two-level one, 0 chooses by size.  Measured on MI355X
+// (ms, three-level / two-level): n = 1024 1.99 / 2.07, 2048 4.32 / 4.39, 4096 10.30 / 10.40,
+// 8192 33.4 / 33.4, 11008 61.2 / 59.7, 14336 107.2 / 106.4.  The K = 1024 products of the explicit Q
+// run at 120 TFLOP/s against 101 for K = 256, but the scheme needs about 15 % more arithmetic (T^T W
+// with K = 1024, a super-block's own columns of Q as one product), and in the factorisation its
+// products arrive in bursts between panel chains, where this GPU gives 100 to 111 TFLOP/s for a
+// product that reaches 127 in a steady stream.
+constexpr int kQrSuperAutoMax = 4096;  // three levels up to this size when the choice is left to the library
+template <typename T>
+static inline int qr_factor_and_form_q(hipStream_t s, T* A, int64_t lda, T* Qout, int64_t ldq, int n,
+                                       const QrWorkspace<T>& ws, int persistent_max_wg = kQrPersistentMaxWg,
+                                       unsigned spin_limit = kQrSpinLimit, int columns_per_round = kQrRoundMax,
+                                       int* report = nullptr, bool carry_updates = true, int super_block = 0) {
+  if (super_block == 0) super_block = n <= kQrSuperAutoMax ? kQrSuper : kBrMax;
+  if (super_block == kQrSuper && columns_per_round == kQrWholePanel && ceil_div64(n, 256) <= persistent_max_wg)
+    return qr_factor_and_form_q_three_level<T>(s, A, lda, Qout, ldq, n, ws, persistent_max_wg, spin_limit, report,
+                                               carry_updates);
+  return qr_factor_and_form_q_two_level<T>(s, A, lda, Qout, ldq, n, ws, persistent_max_wg, spin_limit,
+                                           columns_per_round, report, carry_updates);
 }
 
 }  // namespace soapmi

@@ -4,6 +4,7 @@
 //   abi_probe qr n          QR of a pseudo-random n x n matrix (library-owned workspace), Q checked on the host
 //   abi_probe eigh n        fp64 eigendecomposition of a symmetric n x n matrix, checked on the host
 //   abi_probe eigh n [timed] two-stage   the eigh modes with the two-stage tridiagonalisation
+//   abi_probe qr n [timed] two-level    the qr modes with 256-wide block reflectors only (no super-blocks)
 //   abi_probe qr|eigh n timed   the same call four times, the last three timed, no host check (the
 //                               check is cubic on one core: minutes at n = 11008)
 //
@@ -167,6 +168,10 @@ int main(int argc, char** argv) {
   // a trailing "two-stage" selects the two-stage tridiagonalisation for the eigh modes
   if (argc >= 4 && std::string(argv[1]) == "eigh" && std::string(argv[argc - 1]) == "two-stage") {
     ABI_OK(soapmi_set_option("eigh_algorithm", 2));
+    --argc;
+  }
+  if (argc >= 4 && std::string(argv[1]) == "qr" && std::string(argv[argc - 1]) == "two-level") {
+    ABI_OK(soapmi_set_option("qr_super_block", 256));
     --argc;
   }
   const bool timed_only = argc == 4 && std::string(argv[3]) == "timed";

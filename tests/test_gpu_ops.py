@@ -297,7 +297,7 @@ def test_qr_update_riding_along_with_the_next_panel(size, device):
         _native.call("soapmi_set_option", b"qr_carry_update", 2)
 
 
-@pytest.mark.parametrize("size", [200, 600])
+@pytest.mark.parametrize("size", [200, 600, 1300])
 def test_qr_with_padded_leading_dimensions(size, device):
     """soapmi_qr_f32 called directly with leading dimensions larger than n, for the matrix and for Q:
     the factorisation then cannot use the matrix's own columns as the reflector block of the Q formation."""
@@ -327,6 +327,64 @@ def test_qr_block_reflector_widths(size, device):
     expected_q = oracle.householder_qr(matrix)
     assert relative_l2(factor, expected_q) <= 5e-5
     torch.testing.assert_close(factor.T @ factor, torch.eye(size, device=device), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("size", [300, 1000, 1057, 1312, 2304, 2500])
+def test_qr_super_blocks(size, device):
+    """Three blocking levels (256-column blocks applied inside 1024-column super-blocks, the matrix beyond
+    updated once per super-block with K = 1024) against two: both against LAPACK's Householder QR, and
+    against each other.  Sizes with one, two and three super-blocks, the last one a full 1024 columns,
+    33, 288, 256 and 452 wide (its T factor is then assembled from unequal spans)."""
+    from soap_tp_amd import _native
+    matrix = make_matrix(size, size, seed=SEED + 11 * size)
+    results = {}
+    try:
+        for width in (256, 1024, 0):
+            _native.call("soapmi_set_option", b"qr_super_block", width)
+            factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+            ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
+            results[width] = factor.cpu()
+    finally:
+        _native.call("soapmi_set_option", b"qr_super_block", 0)
+    expected_q = oracle.householder_qr(matrix)
+    for width, factor in results.items():
+        assert relative_l2(factor, expected_q) <= 5e-5, width
+        torch.testing.assert_close(factor.T @ factor, torch.eye(size), rtol=1e-4, atol=1e-4)
+        r = factor.double().T @ matrix.double()
+        assert torch.tril(r, -1).abs().max().item() <= 1e-4 * matrix.abs().max().item() * math.sqrt(size)
+    assert torch.equal(results[0], results[1024])  # sizes up to 4096 take three levels when left to the library
+    with pytest.raises(ValueError):
+        _native.call("soapmi_set_option", b"qr_super_block", 512)
+
+
+@pytest.mark.parametrize("kind", ["paired_columns", "graded", "rank_deficient", "repeated_column"])
+def test_qr_super_blocks_on_hard_matrices(kind, device):
+    """The hard matrices of the test below at a size with two super-blocks, three blocking levels forced."""
+    from soap_tp_amd import _native
+    size = 1400
+    generator = torch.Generator().manual_seed(SEED + 321)
+    matrix = torch.randn(size, size, generator=generator)
+    if kind == "paired_columns":
+        matrix[:, 1::2] = matrix[:, 0::2] + 1e-4 * torch.randn(size, size // 2, generator=generator)
+    elif kind == "graded":
+        matrix = matrix * torch.logspace(0, -12, size)[None, :]
+    elif kind == "rank_deficient":
+        matrix = matrix[:, :40] @ torch.randn(40, size, generator=generator)
+    else:
+        matrix[:, 1:64] = matrix[:, :1]
+    try:
+        _native.call("soapmi_set_option", b"qr_super_block", 1024)
+        factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+        ops.qr_2d_block_cyclic_(column_major(matrix, device), factor, size, BLOCK, GRID)
+    finally:
+        _native.call("soapmi_set_option", b"qr_super_block", 0)
+    q = factor.cpu().double()
+    a = matrix.double()
+    assert torch.isfinite(q).all()
+    assert (q.T @ q - torch.eye(size, dtype=torch.float64)).abs().max().item() <= 2e-5
+    r = torch.triu(q.T @ a)
+    column_norms = a.norm(dim=0).clamp_min(1e-300)
+    assert ((a - q @ r).norm(dim=0) / column_norms).max().item() <= 2e-5  # column-wise backward error
 
 
 @pytest.mark.parametrize("kind", ["paired_columns", "graded", "rank_deficient", "repeated_column"])

@@ -389,6 +389,34 @@ def test_two_stage_eigensolver_at_4096(device):
     assert (spectra[0] - spectra[1]).abs().max().item() <= 1e-6 * spectra[0].abs().max().item()
 
 
+@pytest.mark.parametrize("size,width", [(8192, 1024), (4096, 256)])
+def test_qr_blocking_not_chosen_by_default_at_size(size, width, device):
+    """The QR blocking the library does not pick by itself at this size (three levels above 4096, two
+    up to 4096): orthogonality, triangularity of Q^T W and backward error on a graded matrix."""
+    from soap_tp_amd import _native
+    generator = torch.Generator().manual_seed(4242 + size)
+    matrix = (torch.randn(size, size, generator=generator) * torch.logspace(0, -6, size)[None, :]).to(device)
+    iterate = matrix.T.contiguous().T.clone()  # column-major copy
+    work = iterate.clone()
+    factor = ops.allocate_2d_block_cyclic((size, size), BLOCK, GRID, device=device)
+    try:
+        _native.call("soapmi_set_option", b"qr_super_block", width)
+        ops.qr_2d_block_cyclic_(work, factor, size, BLOCK, GRID)
+    finally:
+        _native.call("soapmi_set_option", b"qr_super_block", 0)
+    del work
+    assert torch.isfinite(factor).all()
+    q, w = factor.double(), iterate.double()
+    identity_error = q.T @ q
+    identity_error.diagonal().sub_(1.0)
+    assert identity_error.abs().max().item() <= 1e-4
+    del identity_error
+    r = q.T @ w
+    assert (torch.tril(r, -1).norm() / w.norm()).item() <= 1e-5
+    backward = w - q @ torch.triu(r)
+    assert (backward.norm(dim=0) / w.norm(dim=0)).max().item() <= 5e-5
+
+
 def test_qr_with_more_workgroups_in_a_launch_than_compute_units(device):
     """n = 16640: a panel launch holds 65 panel workgroups and up to 195 workgroups that update the columns
     behind the panel for the previous one, more than the chip's 256 compute units hold at once.  The
