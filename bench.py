@@ -17,7 +17,9 @@ Stage times come from a second pass over the same schedule that issues the step'
 one by one with event marks between them.  ``roofline`` describes the dominant kernel, the fp32 MFMA
 product behind the four rotation products of a step (algorithmic flops 4 m n (m+n) per step,
 2 m n k per launch), from that pass's events.  After the timed passes one more step is checked
-against the CPU oracle conditionally on the device's bases (``parity_check``).  ``cpu_baseline``
+against the CPU oracle conditionally on the device's bases (``parity_check``: update, moments and both
+Gram matrices; also for every other shape reported and for one parameter per distinct shape of the
+layer).  ``cpu_baseline``
 times the CPU oracle (torch/MKL on the host cores) on a bounded sample of the same workload.
 """
 from __future__ import annotations
@@ -133,25 +135,39 @@ def run_schedule(shape, rank, steps, warmup, device, pool_size=6, interval=10, s
                       detail_total_ms=begin.elapsed_time(end))
 
     if parity:
-        result["parity_check"] = checked_step(gradients[1], state, kwargs, hyper)
+        result["parity_check"] = checked_step(gradients[1], state, kwargs, dict(hyper))
     del state
     return result
 
 
-def checked_step(gradient, state, kwargs, hyper):
+def _lower_to_full(matrix):
+    """The symmetric matrix whose lower triangle (diagonal included) `matrix` holds."""
+    lower = torch.tril(matrix)
+    return lower + torch.tril(matrix, -1).T
+
+
+def checked_step(gradient, state, kwargs, hyper, step_function=None):
     """One more soap_step on the state the timed passes left, compared with the CPU oracle's
-    arithmetic for that step on the same bits, conditionally on the device's bases."""
+    arithmetic for that step on the same bits, conditionally on the device's bases: the update, both
+    moments and both Gram matrices (their lower triangles: the step keeps only those up to date
+    between refreshes).  `step_function(gradient)` makes the step and returns the update; by default it
+    is soap_tp_amd.soap_step on `state`."""
     import soap_tp_amd
     from oracle import soap_oracle as oracle
 
+    if step_function is None:
+        def step_function(g):
+            return soap_tp_amd.soap_step(g, state, **kwargs)
+
     step = int(state["step"]) + 1
     if step % hyper["basis_refresh_interval"] == 0:  # keep the checked step a plain one
-        soap_tp_amd.soap_step(gradient, state, **kwargs)
+        step_function(gradient)
         step += 1
     momentum, variance = state["momentum"].cpu().clone(), state["variance"].cpu().clone()
     q_left, q_right = state["left_basis"].cpu(), state["right_basis"].cpu()
-    update = soap_tp_amd.soap_step(gradient, state, **kwargs).cpu()
-    gradient = gradient.cpu()
+    grams = {side: _lower_to_full(state[f"{side}_preconditioner"].cpu()) for side in ("left", "right")}
+    update = step_function(gradient).cpu()
+    gradient = gradient.cpu().to(torch.float32)
     start = time.perf_counter()
     projected = oracle.rotate(gradient, q_left, q_right, "forward")
     coordinate = oracle.adam_update(projected, momentum, variance, step, hyper["beta1"], hyper["beta2"],
@@ -164,9 +180,14 @@ def checked_step(gradient, state, kwargs, hyper):
 
     errors = {"update": relative(update, expected), "momentum": relative(state["momentum"].cpu(), momentum),
               "variance": relative(state["variance"].cpu(), variance)}
+    for side in ("left", "right"):
+        expected_gram = oracle.gram_ema(grams[side], gradient, hyper["preconditioner_beta"], side)
+        errors[f"{side}_gram"] = relative(torch.tril(state[f"{side}_preconditioner"].cpu()), torch.tril(expected_gram))
+        del expected_gram
     ok = all(math.isfinite(e) and e <= 1e-4 for e in errors.values())
     return {"step": step, "relative_frobenius_error": errors, "tolerance": 1e-4, "ok": ok,
-            "what": "the step after the timed passes against the CPU oracle, given the device's bases",
+            "what": "the step after the timed passes against the CPU oracle, given the device's bases: update, "
+                    "moments, lower triangles of both Gram matrices",
             "cpu_ms": cpu_ms}
 
 
@@ -256,8 +277,28 @@ def run_layer(device, steps=30, rank=64):
     total_ms = begin.elapsed_time(end)
     if not all(bool(torch.isfinite(parameter).all()) for parameter in parameters):
         raise RuntimeError("a parameter of the layer run is not finite")
+    # one more step per distinct shape, checked against the CPU oracle: that parameter alone receives a
+    # gradient, so the wrapper steps only it, and its update is read off the parameter (lr * update)
+    hyper = dict(HYPER)
+    checks = {}
+    lr = optimizer.param_groups[0]["lr"]
+    for shape in dict.fromkeys(shapes):
+        parameter = next(p for p in parameters if tuple(p.shape) == shape)
+        soap_state = optimizer.state[parameter]["soap"]
+
+        def step_function(gradient, parameter=parameter):
+            for other in parameters:
+                other.grad = None
+            before = parameter.detach().clone()
+            parameter.grad = gradient
+            optimizer.step()
+            return (before - parameter.detach()) / lr
+
+        check = checked_step(gradients[shape][1], soap_state, None, hyper, step_function=step_function)
+        # the update passed through p -= lr * update: two more roundings on values of the parameter's size
+        checks[f"{shape[0]}x{shape[1]}"] = check
     flops = sum(5.0 * m * n * (m + n) for m, n in shapes)
-    return {"workload": "4 x 4096x4096, 2 x 4096x14336, 1 x 14336x4096, rank 64, refresh every 10, "
+    return {"parity_check": checks, "workload": "4 x 4096x4096, 2 x 4096x14336, 1 x 14336x4096, rank 64, refresh every 10, "
                         "optimizer wrapper with 2 side streams", "steps": steps,
             "ms_per_layer_step": total_ms / steps, "layer_steps_per_s": steps / (total_ms * 1e-3),
             "initialisation_ms": init_ms, "plain_step_mfma_flops": flops}
@@ -446,13 +487,14 @@ def main():
                                              ((8192, 3584), 128, 100, 5)):
             if shape == args.shape:
                 continue
-            run = run_schedule(shape, rank, steps, interval + 1, device, interval=interval)
+            run = run_schedule(shape, rank, steps, interval + 1, device, interval=interval, parity=True)
             flops = 5.0 * shape[0] * shape[1] * (shape[0] + shape[1])
             plain = run["rotate_ms"] + run["gram_ms"]
             others[f"{shape[0]}x{shape[1]}"] = {
                 "steps": steps, "refresh_every": interval, "steps_per_s": steps / (run["total_ms"] * 1e-3),
                 "plain_step_ms": plain, "refresh_ms": run["refresh_ms"], "initialisation_call_ms": run["init_ms"],
                 "step_mfma_stages_tflops": flops / (plain * 1e-3) / 1e12,
+                "parity_check": run["parity_check"],
             }
         line["other_shapes"] = others
     line["hbm_stages"] = hbm_stages(rows, columns, device)
@@ -470,6 +512,11 @@ def main():
     else:
         line["cpu_baseline"] = None
     print(json.dumps(line))
+    failed = [name for name, entry in line.get("other_shapes", {}).items() if not entry["parity_check"]["ok"]]
+    failed += [f"layer {name}" for name, entry in (line.get("layer") or {}).get("parity_check", {}).items()
+               if not entry["ok"]]
+    if failed:
+        sys.exit(f"bench.py: the checked step disagrees with the CPU oracle for {failed}")
 
 
 if __name__ == "__main__":

@@ -273,6 +273,23 @@ def test_config_8192x3584_refresh_every_5(device, monkeypatch):
         del gram
 
 
+def test_config_4096x4096_full_schedule(device, monkeypatch):
+    """The second benchmark configuration at its full length: 4096 x 4096, rank 64, 50 steps after the
+    initialising call, a refresh every 10 (five refreshes).  Every iteration's update is compared with
+    the oracle given the device's bases, as the reference's end-to-end test follows every iteration
+    of its schedule (tests/unit/test_soap.py:715-817); moments and Gram matrices at the end."""
+    shape = (4096, 4096)
+    gradients = [oracle.low_rank_plus_noise(*shape, 64, seed=SEED + 500 + t) for t in range(51)]
+    updates, state, bases = run_recorded(gradients, device, monkeypatch, interval=10)
+    assert sorted(bases) == [0, 10, 20, 30, 40, 50]
+    assert_conditional_parity(gradients, updates, state, bases, 10)
+    for side in ("left", "right"):
+        q = state[f"{side}_basis"].double()
+        identity_error = q.T @ q
+        identity_error.diagonal().sub_(1.0)
+        assert identity_error.abs().max().item() <= 1e-4
+
+
 LAYER = (("q", (4096, 4096)), ("k", (4096, 4096)), ("v", (4096, 4096)), ("o", (4096, 4096)),
          ("gate", (4096, 14336)), ("up", (4096, 14336)), ("down", (14336, 4096)))
 
