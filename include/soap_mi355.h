@@ -92,6 +92,16 @@ int soapmi_set_option(const char* name, int64_t value);
  * completed so far. */
 int soapmi_device_error_flag(int clear);
 
+/* Failure attribution per optimizer state (the reference throws from the failing call itself,
+ * src/soap_tp/csrc/elpa_bindings.cpp:77-91,149-171, so its caller knows which state failed).
+ * `word` points to one int of device-writable memory that the caller owns and has set to 0 (device
+ * memory, or pinned host memory, which the host can then read without synchronising).  While it is
+ * set, every factorisation the CALLING THREAD enqueues (soapmi_qr_f32, soapmi_power_iteration_qr_f32,
+ * soapmi_refresh_f32, soapmi_eigh_f64/f32, soapmi_initialize_basis_f32) raises *word to 1 instead of
+ * the device's word when one of its kernels gives up; NULL restores the per-device word.  The word
+ * must stay valid until the kernels enqueued while it was set have finished. */
+int soapmi_set_status_word(int* word);
+
 /* ---- Gram preconditioner EMA ---------------------------------------------------------- */
 
 /* P <- lerp(P, G G^T, 1-beta) (side 0, P is rows x rows) or lerp(P, G^T G, 1-beta) (side 1,

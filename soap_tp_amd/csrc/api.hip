@@ -129,6 +129,21 @@ static int device_report(int** out) {
   return kOk;
 }
 
+// A caller-owned status word (device-writable memory: device memory or pinned host memory) that the
+// factorisations enqueued by the calling thread raise instead of the per-device report word, so that
+// a failure can be told apart per optimizer state: soapmi_set_status_word.
+static thread_local int* t_status_word = nullptr;
+
+// Where a factorisation's last kernel reports a failure: the caller's status word if one is set for
+// this thread, else the device's report word.
+static int failure_report(int** out) {
+  if (t_status_word) {
+    *out = t_status_word;
+    return kOk;
+  }
+  return device_report(out);
+}
+
 // Persistent kernels (the QR panel kernel, the tridiagonalisation's column kernel) wait inside the
 // kernel for messages from the other workgroups of their launch, so all workgroups of a launch must
 // be resident together.  One launch always is (at most 128 workgroups on 256 compute units), but
@@ -139,6 +154,21 @@ static int device_report(int** out) {
 // budget.  Host-side enqueueing of factorisations is serialised per device for the time of the
 // call, which keeps the bookkeeping simple; nothing here synchronises the host with the device.
 static std::atomic<int> g_persistent_budget{256};
+
+// Compute units of the current device (looked up once per device): a persistent workgroup of the
+// panel kernels takes a whole one, so neither the budget nor one launch may exceed their number on
+// a partitioned or masked device.
+static int compute_unit_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int count = cached[dev].load();
+  if (count == 0) {
+    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || count <= 0) count = 256;
+    cached[dev].store(count);
+  }
+  return count;
+}
 
 struct PersistentLease {
   hipEvent_t done = nullptr;
@@ -174,7 +204,7 @@ class PersistentGuard {
     ledger_ = &g_ledger[dev];
     ledger_->enqueue.lock();
     stream_ = stream;
-    const int budget = g_persistent_budget.load();
+    const int budget = std::min(g_persistent_budget.load(), compute_unit_count());
     int in_flight = 0;
     PersistentLease* free_slot = nullptr;
     for (PersistentLease& lease : ledger_->leases) {
@@ -276,6 +306,13 @@ static int check_adam_args(int64_t step, double beta1, double beta2, double eps)
 
 using namespace soapmi;
 
+// Workspace of an eigensolve whichever tridiagonalisation is selected when the call is made: the
+// option can change between a caller's size query and its call.
+template <typename T>
+static size_t eigh_workspace_bytes_any(int64_t n) {
+  return std::max(eigh_workspace_bytes<T>(n, kEighOneStage), eigh_workspace_bytes<T>(n, kEighTwoStage));
+}
+
 template <typename T>
 static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_t ldq, void* workspace,
                       size_t workspace_bytes, void* stream) {
@@ -283,7 +320,7 @@ static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_
   SOAPMI_REQUIRE(n > 0, "matrix dimensions and block size must be positive");
   SOAPMI_REQUIRE(lda >= n && ldq >= n, "leading dimensions are too small");
   SOAPMI_REQUIRE(n <= 32768, "matrix size %lld exceeds the supported maximum 32768", (long long)n);
-  const int algorithm = g_eigh_algorithm.load();
+  const int algorithm = g_eigh_algorithm.load();  // (read once: everything below uses this value)
   const size_t need = eigh_workspace_bytes<T>(n, algorithm);
   void* ws = nullptr;
   int rc = resolve_workspace(workspace, workspace_bytes, need, &ws);
@@ -292,7 +329,7 @@ static int eigh_entry(T* a, T* eigenvalues, T* q, int64_t n, int64_t lda, int64_
   EighWorkspace<T> ews;
   eigh_workspace_layout<T>(w, n, &ews, algorithm);
   int* report = nullptr;
-  rc = device_report(&report);
+  rc = failure_report(&report);
   if (rc) return rc;
   PersistentGuard guard;
   rc = guard.acquire((hipStream_t)stream, (int)ceil_div64(n, 256));
@@ -318,10 +355,14 @@ int soapmi_device_error_flag(int clear) {
   int* report = nullptr;
   int rc = device_report(&report);
   if (rc) return rc;
-  volatile int* word = report;
-  const int raised = *word != 0 ? 1 : 0;
-  if (clear) *word = 0;
-  return raised;
+  // (one exchange: a kernel that raises the word between a read and a separate clearing store would be lost)
+  const int value = clear ? __atomic_exchange_n(report, 0, __ATOMIC_ACQ_REL) : __atomic_load_n(report, __ATOMIC_ACQUIRE);
+  return value != 0 ? 1 : 0;
+}
+
+int soapmi_set_status_word(int* word) {
+  t_status_word = word;
+  return kOk;
 }
 
 int soapmi_set_option(const char* name, int64_t value) {
@@ -780,13 +821,14 @@ int soapmi_qr_f32(float* matrix, float* q, int64_t n, int64_t ldmatrix, int64_t 
   QrWorkspace<float> qws;
   qr_workspace_layout<float>(w, n, &qws);
   int* report = nullptr;
-  rc = device_report(&report);
+  rc = failure_report(&report);
   if (rc) return rc;
   PersistentGuard guard;
   rc = guard.acquire((hipStream_t)stream, (int)ceil_div64(n, 256));
   if (rc) return rc;
   rc = qr_factor_and_form_q<float>((hipStream_t)stream, matrix, ldmatrix, q, ldq, (int)n, qws,
-                                   g_qr_persistent_max_wg.load(), g_message_spin_limit.load(),
+                                   std::min(g_qr_persistent_max_wg.load(), compute_unit_count()),
+                                   g_message_spin_limit.load(),
                                    g_qr_columns_per_round.load(), report, g_qr_carry_update.load() != 0,
                                    g_qr_super_block.load());
   const int rc_release = guard.release();
@@ -905,8 +947,7 @@ int soapmi_refresh_f32(float* momentum, int64_t ldm, float* variance, int64_t ld
 // ---- eigensolver ------------------------------------------------------------------------------
 
 size_t soapmi_eigh_workspace_bytes(int64_t n, int element_bytes) {
-  const int algorithm = g_eigh_algorithm.load();
-  return element_bytes == 8 ? eigh_workspace_bytes<double>(n, algorithm) : eigh_workspace_bytes<float>(n, algorithm);
+  return element_bytes == 8 ? eigh_workspace_bytes_any<double>(n) : eigh_workspace_bytes_any<float>(n);
 }
 
 int soapmi_eigh_f64(double* a, double* eigenvalues, double* q, int64_t n, int64_t lda, int64_t ldq,
@@ -925,12 +966,12 @@ size_t soapmi_initialize_basis_workspace_bytes(int64_t n, int implementation) {
     w.take<double>((size_t)n * n);
     w.take<double>((size_t)n * n);
     w.take<double>((size_t)n);
-    w.take<char>(eigh_workspace_bytes<double>(n, g_eigh_algorithm.load()));
+    w.take<char>(eigh_workspace_bytes_any<double>(n));
   } else {
     w.take<float>((size_t)n * n);
     w.take<float>((size_t)n * n);
     w.take<float>((size_t)n);
-    w.take<char>(eigh_workspace_bytes<float>(n, g_eigh_algorithm.load()));
+    w.take<char>(eigh_workspace_bytes_any<float>(n));
   }
   return w.total();
 }
@@ -957,7 +998,7 @@ int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* ei
     double* a64 = w.take<double>((size_t)n * n);
     double* z64 = w.take<double>((size_t)n * n);
     double* w64 = w.take<double>((size_t)n);
-    const size_t eb = eigh_workspace_bytes<double>(n, g_eigh_algorithm.load());
+    const size_t eb = eigh_workspace_bytes_any<double>(n);
     char* ebuf = w.take<char>(eb);
     // work <- -P (both triangles), then its float64 copy, as factorizations.py:500-507 stages them
     hipLaunchKernelGGL((sym_convert_kernel<float, float>), tiles, dim3(256), 0, s, p, ldp, work, ldw, (int)n, -1.0f, 0.0f);
@@ -972,7 +1013,7 @@ int soapmi_initialize_basis_f32(const float* p, float* q, float* work, float* ei
     float* a32 = w.take<float>((size_t)n * n);
     float* z32 = w.take<float>((size_t)n * n);
     float* w32 = w.take<float>((size_t)n);
-    const size_t eb = eigh_workspace_bytes<float>(n, g_eigh_algorithm.load());
+    const size_t eb = eigh_workspace_bytes_any<float>(n);
     char* ebuf = w.take<char>(eb);
     hipLaunchKernelGGL((sym_convert_kernel<float, float>), tiles, dim3(256), 0, s, p, ldp, a32, n, (int)n, 1.0f, 1e-30f);
     SOAPMI_LAUNCH_CHECK();

@@ -37,6 +37,44 @@ def raise_on_device_error(device) -> None:
             )
 
 
+def new_status_word() -> Tensor:
+    """One zeroed int32 of pinned host memory: kernels raise it, the host reads it without synchronising."""
+    return torch.zeros(1, dtype=torch.int32, pin_memory=True)
+
+
+class reporting_to:
+    """While active, factorisations enqueued by this thread report a failure on the device in the
+    given pinned int32 tensor instead of the device-wide flag (``None``: no change)."""
+
+    def __init__(self, status: Optional[Tensor]):
+        if status is not None and (status.dtype != torch.int32 or status.numel() < 1 or not status.is_pinned()):
+            raise ValueError("status must be a pinned int32 tensor with at least one element.")
+        self.status = status
+
+    def __enter__(self):
+        if self.status is not None:
+            _native.call("soapmi_set_status_word", self.status.data_ptr())
+        return self
+
+    def __exit__(self, *exc):
+        if self.status is not None:
+            _native.call("soapmi_set_status_word", 0)
+        return False
+
+
+def raise_on_state_error(state) -> None:
+    """Raise if a factorisation of THIS state (its initialisation or one of its refreshes) failed on
+    the device: the state's status word stays raised, so every later step of the state raises too,
+    while other states on the device go on.  Reads pinned host memory, no synchronisation."""
+    status = state.get("status") if hasattr(state, "get") else None
+    if isinstance(status, Tensor) and int(status[0]) != 0:
+        raise RuntimeError(
+            "a QR or eigensolver kernel of this optimizer state gave up waiting for a message from another "
+            "workgroup; its bases are NaN-poisoned and the state is invalid. Re-initialise the state (or "
+            "restore a checkpoint)."
+        )
+
+
 def require_device_tensor(name: str, tensor: Tensor) -> None:
     """The kernels run on the GPU only; same rule and wording as the reference's backend check
     (src/soap_tp/ops/factorizations.py:33-48 with backend 'rocm')."""

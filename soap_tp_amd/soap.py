@@ -11,6 +11,9 @@ Same signature, state dictionary and sequencing as the reference orchestrator
   ``step % basis_refresh_interval == 0``, refresh the bases and transport the optimizer state
   (:457-471).
 
+Beyond the reference's keys the state holds ``"status"``: one int32 of pinned host memory that a
+factorisation kernel of this state raises if it gives up on the device (see ``soap_tp_amd.ops._common``).
+
 The default path issues three library calls per step (update, left Gram, right Gram; plus one
 on refresh steps) on torch's current stream and never synchronises.  When a binding object is
 injected (``slate_binding`` / ``elpa_binding``) or ``SOAP_PROFILE`` is set, the step runs op by
@@ -37,8 +40,8 @@ from .ops import (
     update_left_preconditioner_2d_block_cyclic_,
     update_right_preconditioner_2d_block_cyclic_,
 )
-from .ops._common import (native_call, native_library, raise_on_device_error, require_device_tensor, scratch,
-                          stream_of)
+from .ops._common import (native_call, native_library, new_status_word, raise_on_device_error,
+                          raise_on_state_error, reporting_to, require_device_tensor, scratch, stream_of)
 from .ops._utils import current_world
 
 STATE_BUFFERS = (
@@ -146,8 +149,14 @@ def soap_step(
     require_device_tensor("gradient_shard", gradient_shard)
     mirror = preconditioner_storage == "full"
     device = gradient_shard.device
+    # A factorisation kernel that failed on the device: this state's own word first (set by its
+    # initialisation and refreshes, and left raised, so a poisoned state raises on every later step while
+    # other states go on), then the device-wide word that factorisations enqueued without one raise.
+    raise_on_state_error(state)
     raise_on_device_error(device)
     initializing = "left_basis" not in state
+    if "status" not in state:  # (a state restored from a checkpoint comes without one)
+        state["status"] = new_status_word()
 
     if initializing:
         for name, shape in _state_shapes(rows, columns).items():
@@ -178,10 +187,11 @@ def soap_step(
     if initializing:
         update_preconditioners("")
         for side, size in (("left", rows), ("right", columns)):
-            initialize_basis_2d_block_cyclic_(
-                state[f"{side}_preconditioner"], state[f"{side}_basis"], state[f"{side}_work"],
-                torch.empty(size, dtype=torch.float32, device=device), size, block_size,
-                process_grid_shape, implementation=basis_implementation, elpa_binding=elpa_binding)
+            with reporting_to(state["status"]):
+                initialize_basis_2d_block_cyclic_(
+                    state[f"{side}_preconditioner"], state[f"{side}_basis"], state[f"{side}_work"],
+                    torch.empty(size, dtype=torch.float32, device=device), size, block_size,
+                    process_grid_shape, implementation=basis_implementation, elpa_binding=elpa_binding)
             _profile.dump(f"{side}_basis", profile_step, state[f"{side}_basis"])
         state["step"] = 0
         zero_update = torch.zeros_like(gradient)
@@ -219,11 +229,12 @@ def soap_step(
 
     update_preconditioners("_after_step")
     if step % basis_refresh_interval == 0:
-        refresh_bases_and_transport_optimizer_state_(
-            state["momentum"], state["variance"], state["left_preconditioner"],
-            state["right_preconditioner"], state["left_basis"], state["right_basis"],
-            state["left_work"], state["right_work"], global_shape, block_size, process_grid_shape,
-            slate_binding=slate_binding, symmetrize=not mirror)
+        with reporting_to(state["status"]):
+            refresh_bases_and_transport_optimizer_state_(
+                state["momentum"], state["variance"], state["left_preconditioner"],
+                state["right_preconditioner"], state["left_basis"], state["right_basis"],
+                state["left_work"], state["right_work"], global_shape, block_size, process_grid_shape,
+                slate_binding=slate_binding, symmetrize=not mirror)
     if profiling:
         _profile.dump("left_basis_after_step", profile_step, state["left_basis"])
         _profile.dump("right_basis_after_step", profile_step, state["right_basis"])

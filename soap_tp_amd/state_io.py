@@ -4,7 +4,8 @@ The state holds eight strided column-major matrices (``zeros((cols, ld)).T`` vie
 src/soap_tp/ops/_utils.py:159-189) and the integer step (src/soap_tp/soap.py:166-175).  Serialisers
 that only keep contiguous data (safetensors, ``tensor.contiguous()`` round trips, dtype casts) lose
 that layout, and ``soap_step`` rejects buffers that are not column-major.  ``pack_state`` therefore
-stores every buffer as the contiguous ``(cols, rows)`` transpose together with its logical shape, and
+stores every buffer as the contiguous ``(cols, rows)`` transpose together with its logical shape (the
+Gram matrices symmetrised from their lower triangle, the one ``soap_step`` keeps current), and
 ``unpack_state`` rebuilds the exact layout (``stride == (1, max(1, rows))``) on the target device and
 checks shapes, dtype and mutual consistency before the state is used again.  The reference has no
 such helper; its .gitignore:18-20 only anticipates ``.pt`` checkpoints.
@@ -65,6 +66,10 @@ def validate_state(state: Mapping[str, Any], global_shape: Optional[Tuple[int, i
     step = state["step"]
     if isinstance(step, bool) or not isinstance(step, int) or step < 0:
         raise ValueError(f"state['step'] must be a non-negative int, got {step!r}.")
+    status = state.get("status")
+    if isinstance(status, Tensor) and int(status[0]) != 0:
+        raise ValueError("a factorisation of this state failed on the device (state['status'] is raised): its "
+                         "bases are NaN-poisoned.")
     return rows, columns
 
 
@@ -77,7 +82,14 @@ def pack_state(state: Mapping[str, Any]) -> Dict[str, Any]:
     packed: Dict[str, Any] = {"format_version": FORMAT_VERSION, "initialised": True, "rows": rows,
                               "columns": columns, "step": int(state["step"])}
     for name in STATE_BUFFERS:
-        packed[name] = state[name].detach().T.contiguous()
+        buffer = state[name].detach()
+        if name.endswith("_preconditioner"):
+            # soap_step keeps only the lower triangle of a Gram matrix up to date between refreshes
+            # (preconditioner_storage="lower"); a saved state has both triangles valid, as the
+            # reference's state contract asks (src/soap_tp/ops/factorizations.py:378)
+            packed[name] = (torch.tril(buffer) + torch.tril(buffer, -1).T).contiguous()
+        else:
+            packed[name] = buffer.T.contiguous()
     return packed
 
 

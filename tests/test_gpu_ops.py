@@ -462,10 +462,11 @@ def test_lost_messages_poison_the_result_instead_of_hanging(device):
 
 def test_soap_step_raises_after_a_factorisation_failed_on_the_device(device):
     """A refresh whose QR gives up (spin limit 0, several workgroups) leaves NaN-poisoned bases; the
-    next call of soap_step on that device must raise instead of computing with them.  If every
-    message happened to be there at the first poll nothing failed and nothing may be raised."""
+    next call of soap_step on that state must raise instead of computing with them, and so must
+    every call after it.  If every message happened to be there at the first poll nothing failed
+    and nothing may be raised.  The failure is the state's own: the device-wide flag stays down."""
     import soap_tp_amd
-    from soap_tp_amd import _native
+    from soap_tp_amd import _native, state_io
     shape = (700, 520)
     generator = torch.Generator().manual_seed(SEED + 79)
     state = {}
@@ -480,13 +481,69 @@ def test_soap_step_raises_after_a_factorisation_failed_on_the_device(device):
     finally:
         _native.call("soapmi_set_option", b"message_spin_limit", 1 << 22)
     poisoned = bool(torch.isnan(state["left_basis"]).any() or torch.isnan(state["right_basis"]).any())
+    assert bool(state["status"][0] != 0) == poisoned
     gradient = torch.randn(*shape, generator=generator).to(device)
     if poisoned:
-        with pytest.raises(RuntimeError, match="gave up waiting"):
-            soap_tp_amd.soap_step(gradient, state, **kwargs)
+        for _ in range(2):
+            with pytest.raises(RuntimeError, match="gave up waiting"):
+                soap_tp_amd.soap_step(gradient, state, **kwargs)
+        with pytest.raises(ValueError, match="failed on the device"):
+            state_io.pack_state(state)
     else:
         soap_tp_amd.soap_step(gradient, state, **kwargs)
-    assert not _native.device_error_flag(clear=True)  # raising cleared it
+    assert not _native.device_error_flag(clear=True)
+
+
+def test_a_failed_factorisation_is_attributed_to_its_state(device):
+    """Two parameters on one device.  One parameter's refresh runs with no patience for messages (spin
+    limit 0 during that call only; every kernel still exits normally).  Only that parameter's state
+    may raise afterwards; the other one keeps stepping, through its own refreshes too, and its
+    results equal those of a run in which nothing failed."""
+    import soap_tp_amd
+    from soap_tp_amd import _native
+    shapes = {"a": (700, 520), "b": (520, 700)}
+    kwargs = {name: dict(global_shape=shape, shard_dim=1, block_size=128, process_grid_shape=GRID,
+                         basis_refresh_interval=2) for name, shape in shapes.items()}
+    generator = torch.Generator().manual_seed(SEED + 81)
+    gradients = {name: [torch.randn(*shape, generator=generator).to(device) for _ in range(7)]
+                 for name, shape in shapes.items()}
+
+    def run(fail):
+        states = {"a": {}, "b": {}}
+        updates = []
+        raised = False
+        for t in range(7):
+            for name in ("a", "b"):
+                failing = fail and name == "a" and t == 2  # the first refresh of parameter a
+                try:
+                    if failing:
+                        _native.call("soapmi_set_option", b"message_spin_limit", 0)
+                    try:
+                        update = soap_tp_amd.soap_step(gradients[name][t], states[name], **kwargs[name])
+                    except RuntimeError as error:
+                        assert name == "a" and t > 2 and "gave up waiting" in str(error)
+                        raised = True
+                        continue
+                    if failing:
+                        torch.cuda.synchronize()
+                finally:
+                    if failing:
+                        _native.call("soapmi_set_option", b"message_spin_limit", 1 << 22)
+                if name == "b":
+                    updates.append(update.cpu())
+        return states, updates, raised
+
+    assert not _native.device_error_flag(clear=True)
+    clean_states, clean_updates, clean_raised = run(fail=False)
+    assert not clean_raised
+    states, updates, raised = run(fail=True)
+    poisoned = bool(torch.isnan(states["a"]["left_basis"]).any() or torch.isnan(states["a"]["right_basis"]).any())
+    assert raised == poisoned  # (all messages there at the first poll: nothing failed, nothing raised)
+    assert int(states["b"]["status"][0]) == 0 and int(states["b"]["step"]) == 6
+    assert len(updates) == len(clean_updates) == 7
+    for update, clean in zip(updates, clean_updates):
+        assert torch.equal(update, clean)
+    assert not _native.device_error_flag(clear=True)  # the device-wide word was never involved
 
 
 @pytest.mark.parametrize("budget", [256, 20])

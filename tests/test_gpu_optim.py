@@ -144,16 +144,26 @@ def test_checkpoint_round_trip_continues_bit_exactly(device):
 def test_state_helpers_on_device(device, tmp_path):
     shape = (24, 40)
     state = {}
-    gradients = [oracle.low_rank_plus_noise(*shape, 4, seed=s).to(device) for s in range(4)]
+    gradients = [oracle.low_rank_plus_noise(*shape, 4, seed=s).to(device) for s in range(5)]
     kwargs = dict(global_shape=shape, shard_dim=1, block_size=8, process_grid_shape=(1, 1), basis_refresh_interval=2)
     for gradient in gradients[:3]:
         soap_tp_amd.soap_step(gradient, state, **kwargs)
+    # saved between two refreshes (step 2 refreshed, step 3 has not happened): the state's upper
+    # triangles are stale, the file's Gram matrices must be symmetric all the same
+    soap_tp_amd.soap_step(gradients[3], state, **kwargs)
     state_io.save_state(state, tmp_path / "state.pt")
+    raw = torch.load(tmp_path / "state.pt", weights_only=True)
+    for side in ("left", "right"):
+        saved = raw[f"{side}_preconditioner"]
+        assert torch.equal(saved, saved.T)
+        assert torch.equal(torch.tril(saved), torch.tril(state[f"{side}_preconditioner"].cpu()))
+        assert not torch.equal(state[f"{side}_preconditioner"], state[f"{side}_preconditioner"].T)
     clone = state_io.load_state(tmp_path / "state.pt", device=device)
     assert state_io.validate_state(clone, shape) == shape
-    a = soap_tp_amd.soap_step(gradients[3], state, **kwargs)
-    b = soap_tp_amd.soap_step(gradients[3], clone, **kwargs)
-    assert torch.equal(a, b) and clone["step"] == state["step"] == 3
+    a = soap_tp_amd.soap_step(gradients[4], state, **kwargs)  # a refresh step: reads the Gram matrices
+    b = soap_tp_amd.soap_step(gradients[4], clone, **kwargs)
+    assert torch.equal(a, b) and clone["step"] == state["step"] == 4
+    assert torch.equal(clone["left_basis"], state["left_basis"]) and torch.equal(clone["right_basis"], state["right_basis"])
 
 
 def test_profile_dump_diffs_clean_against_the_oracle(device, monkeypatch, capfd, tmp_path):

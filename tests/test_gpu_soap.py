@@ -122,7 +122,7 @@ def test_soap_step_matches_oracle_and_golden_trajectory(shape, implementation, s
     assert state["step"] == len(gradients) - 1 == expected_state["step"]
     assert relative_l2(_full(state["left_preconditioner"]), expected_state["left_preconditioner"]) <= TOL
     assert relative_l2(_full(state["right_preconditioner"]), expected_state["right_preconditioner"]) <= TOL
-    assert sorted(state) == sorted(list(soap_module.STATE_BUFFERS) + ["step"])
+    assert sorted(state) == sorted(list(soap_module.STATE_BUFFERS) + ["step", "status"])  # the reference's keys + the failure word
     for name in soap_module.STATE_BUFFERS:
         assert state[name].stride(0) == 1 and state[name].dtype == torch.float32
 

@@ -34,8 +34,31 @@ def test_pack_unpack_round_trip_restores_values_and_layout(pad):
     restored = state_io.unpack_state(packed)
     assert restored["step"] == 4
     for name in state_io.STATE_BUFFERS:
-        assert torch.equal(restored[name], state[name])
+        assert torch.equal(restored[name], _saved_form(name, state[name]))
         assert restored[name].stride() == (1, max(1, state[name].size(0)))
+
+
+def _saved_form(name, tensor):
+    """What a saved state holds for a buffer: Gram matrices symmetrised from their lower triangle."""
+    if name.endswith("_preconditioner"):
+        return torch.tril(tensor) + torch.tril(tensor, -1).T
+    return tensor
+
+
+def test_saved_gram_matrices_are_symmetric_whatever_the_upper_triangle_held():
+    """soap_step keeps only the lower triangle of the Gram matrices current between refreshes; a saved
+    state must have both triangles valid (src/soap_tp/ops/factorizations.py:378)."""
+    state = _state(rows=6, columns=9)
+    for side in ("left", "right"):
+        matrix = state[f"{side}_preconditioner"]
+        matrix.copy_(torch.tril(matrix) + torch.tril(matrix, -1).T)
+    expected = {side: state[f"{side}_preconditioner"].clone() for side in ("left", "right")}
+    for side in ("left", "right"):  # a stale upper triangle
+        state[f"{side}_preconditioner"].add_(torch.triu(torch.full_like(expected[side], 7.0), 1))
+    restored = state_io.unpack_state(state_io.pack_state(state))
+    for side in ("left", "right"):
+        assert torch.equal(restored[f"{side}_preconditioner"], expected[side])
+        assert torch.equal(restored[f"{side}_preconditioner"], restored[f"{side}_preconditioner"].T)
 
 
 def test_save_load_round_trip_uses_a_safe_loader(tmp_path):
@@ -47,7 +70,7 @@ def test_save_load_round_trip_uses_a_safe_loader(tmp_path):
     assert loaded is target and "stale" not in target
     assert state_io.validate_state(loaded) == (3, 5)
     for name in state_io.STATE_BUFFERS:
-        assert torch.equal(loaded[name], state[name])
+        assert torch.equal(loaded[name], _saved_form(name, state[name]))
     # the file holds tensors and plain scalars only
     raw = torch.load(path, weights_only=True)
     assert raw["rows"] == 3 and raw["columns"] == 5 and raw["step"] == 4

@@ -54,6 +54,29 @@ def test_static_scratch_entry_point_equals_workspace_entry_point(device):
             assert torch.equal(expected, actual), shape
 
 
+def test_static_scratch_entry_point_allocates_no_device_memory(device):
+    """What the entry point exists for: with inputs and outputs in place, the free device memory the
+    driver reports is the same before and after its calls (sizes this process has not run before, so
+    nothing is served from a cache; the library's own grow-only scratch is not involved either)."""
+    stream = torch.cuda.current_stream(device).cuda_stream
+    prepared = []
+    for shape, seed in (((768, 1280), SEED + 920), ((96, 72), SEED + 930)):
+        gradient, q_left, q_right, momentum, variance = _inputs(*shape, seed, device)
+        prepared.append((gradient, q_left, q_right, momentum, variance, torch.empty_like(gradient)))
+    torch.cuda.synchronize(device)
+    free_before, _ = torch.cuda.mem_get_info(device)
+    for gradient, q_left, q_right, momentum, variance, update in prepared:
+        rows, columns = gradient.shape
+        _native.call("soapmi_rotate_adam_rotate_static_f32", gradient.data_ptr(), gradient.stride(0),
+                     update.data_ptr(), update.stride(0), q_left.data_ptr(), q_left.stride(1), q_right.data_ptr(),
+                     q_right.stride(1), momentum.data_ptr(), momentum.stride(1), variance.data_ptr(),
+                     variance.stride(1), rows, columns, 2, 0.9, 0.95, 1e-8, stream)
+    torch.cuda.synchronize(device)
+    free_after, _ = torch.cuda.mem_get_info(device)
+    assert free_after == free_before
+    assert all(torch.isfinite(item[5]).all() for item in prepared)
+
+
 def test_static_scratch_entry_point_rejects_what_does_not_fit(device):
     stream = torch.cuda.current_stream(device).cuda_stream
     rows, columns = 2048, 2049  # one column more than the array holds
