@@ -2,6 +2,7 @@
 #include <stdarg.h>
 
 #include <atomic>
+#include <condition_variable>
 #include <mutex>
 
 #include "../../include/soap_mi355.h"
@@ -151,8 +152,8 @@ static int failure_report(int** out) {
 // chip while waiting for workgroups that find no free slot.  The library therefore keeps, per
 // device, the workgroup counts of the factorisations that may still be running (an event marks the
 // end of each) and makes a new one wait, on the device, for earlier ones until the sum fits the
-// budget.  Host-side enqueueing of factorisations is serialised per device for the time of the
-// call, which keeps the bookkeeping simple; nothing here synchronises the host with the device.
+// budget.  Nothing here synchronises the host with the device; host threads that enqueue
+// factorisations at the same time only share the bookkeeping.
 static std::atomic<int> g_persistent_budget{256};
 
 // Compute units of the current device (looked up once per device): a persistent workgroup of the
@@ -173,10 +174,12 @@ static int compute_unit_count() {
 struct PersistentLease {
   hipEvent_t done = nullptr;
   int workgroups = 0;
-  bool active = false;
+  bool active = false;    // taken by a factorisation that may still be running
+  bool recorded = false;  // its end has been recorded in `done` (false while its launches are still being enqueued)
 };
 struct PersistentLedger {
-  std::recursive_mutex enqueue;
+  std::mutex mutex;               // guards the leases; held for the bookkeeping only, not while launching
+  std::condition_variable changed;  // a lease was recorded or given up
   PersistentLease leases[32];
 };
 static PersistentLedger g_ledger[64];
@@ -187,13 +190,16 @@ class PersistentGuard {
   PersistentGuard(const PersistentGuard&) = delete;
   PersistentGuard& operator=(const PersistentGuard&) = delete;
   ~PersistentGuard() {
-    if (ledger_) {
-      if (lease_) lease_->active = false;  // left without release(): nothing was recorded
-      ledger_->enqueue.unlock();
+    if (ledger_ && lease_) {  // left without release(): nothing was recorded
+      std::lock_guard<std::mutex> lock(ledger_->mutex);
+      lease_->active = false;
+      ledger_->changed.notify_all();
     }
   }
   // Call before the first launch of a factorisation whose persistent kernels have up to `workgroups`
-  // workgroups, on the stream it will run on.
+  // workgroups, on the stream it will run on.  Threads may enqueue factorisations side by side: one
+  // that has to wait for a factorisation another thread is still enqueueing waits on the host until
+  // that one's end has been recorded, then on the device for the recorded event.
   int acquire(hipStream_t stream, int workgroups) {
     int dev = 0;
     SOAPMI_HIP(hipGetDevice(&dev));
@@ -202,34 +208,44 @@ class PersistentGuard {
       return kRuntimeError;
     }
     ledger_ = &g_ledger[dev];
-    ledger_->enqueue.lock();
     stream_ = stream;
     const int budget = std::min(g_persistent_budget.load(), compute_unit_count());
-    int in_flight = 0;
-    PersistentLease* free_slot = nullptr;
-    for (PersistentLease& lease : ledger_->leases) {
-      if (lease.active && hipEventQuery(lease.done) == hipSuccess) lease.active = false;
-      if (lease.active) in_flight += lease.workgroups;
-      else if (!free_slot) free_slot = &lease;
-    }
-    (void)hipGetLastError();  // hipEventQuery reports "not ready" through the error state
-    // Wait (on the device) for earlier factorisations until this one fits; also when no slot is
-    // free.  A factorisation this one waits for never runs beside it, so the two together hold at
-    // most the larger of their counts at any time: the waited-for entry is folded into this one.
+    std::unique_lock<std::mutex> lock(ledger_->mutex);
     int held = workgroups;
-    for (PersistentLease& lease : ledger_->leases) {
-      if (in_flight + held <= budget && free_slot) break;
-      if (!lease.active) continue;
-      SOAPMI_HIP(hipStreamWaitEvent(stream, lease.done, 0));
-      in_flight -= lease.workgroups;
-      if (lease.workgroups > held) held = lease.workgroups;
-      lease.active = false;
-      if (!free_slot) free_slot = &lease;
+    for (;;) {
+      int in_flight = 0;
+      PersistentLease* free_slot = nullptr;
+      for (PersistentLease& lease : ledger_->leases) {
+        if (lease.active && lease.recorded && hipEventQuery(lease.done) == hipSuccess) lease.active = false;
+        if (lease.active) in_flight += lease.workgroups;
+        else if (!free_slot) free_slot = &lease;
+      }
+      (void)hipGetLastError();  // hipEventQuery reports "not ready" through the error state
+      if ((in_flight + held <= budget || in_flight == 0) && free_slot) {  // (one larger than the budget runs alone)
+        lease_ = free_slot;
+        break;
+      }
+      // Wait for one earlier factorisation and look again.  A factorisation this one waits for never
+      // runs beside it, so the two together hold at most the larger of their counts at any time: the
+      // waited-for entry is folded into this one.
+      PersistentLease* recorded = nullptr;
+      for (PersistentLease& lease : ledger_->leases)
+        if (lease.active && lease.recorded) {
+          recorded = &lease;
+          break;
+        }
+      if (recorded) {
+        SOAPMI_HIP(hipStreamWaitEvent(stream, recorded->done, 0));
+        if (recorded->workgroups > held) held = recorded->workgroups;
+        recorded->active = false;
+      } else {
+        ledger_->changed.wait(lock);  // every active one is still being enqueued by another thread
+      }
     }
-    lease_ = free_slot;
     if (!lease_->done) SOAPMI_HIP(hipEventCreateWithFlags(&lease_->done, hipEventDisableTiming));
     lease_->workgroups = held;
     lease_->active = true;
+    lease_->recorded = false;
     return kOk;
   }
   // Call after the last launch of the factorisation.
@@ -238,11 +254,15 @@ class PersistentGuard {
     PersistentLease* lease = lease_;
     lease_ = nullptr;
     hipError_t e = hipEventRecord(lease->done, stream_);
+    std::lock_guard<std::mutex> lock(ledger_->mutex);
     if (e != hipSuccess) {
       lease->active = false;
+      ledger_->changed.notify_all();
       set_error("hipEventRecord failed: %s", hipGetErrorString(e));
       return kRuntimeError;
     }
+    lease->recorded = true;
+    ledger_->changed.notify_all();
     return kOk;
   }
 

@@ -15,10 +15,12 @@ ground truth (tests/reference/soap.py:46-143, :145-345):
 
 Independent parameters are issued round-robin on a small pool of side streams (default priority)
 forked from and joined back into the current stream, so the launch-bound steps of small matrices
-overlap each other and the tails of large ones.
+overlap each other and the tails of large ones.  The step that initialises states (two eigensolves
+per matrix, tens of thousands of launches each) issues them from one host thread per side stream.
 """
 from __future__ import annotations
 
+import threading
 from typing import Any, Dict, Iterable, List, Optional, Tuple
 
 import torch
@@ -149,6 +151,34 @@ class SOAP(torch.optim.Optimizer):
             self._streams[device] = [torch.cuda.Stream(device=device) for _ in range(self._stream_count)]
         return self._streams[device]
 
+    def _uninitialised(self, p: Tensor) -> bool:
+        """A parameter that soap_step preconditions and whose state has not been initialised yet."""
+        preconditioned = p.ndim > 2 or (p.ndim == 2 and p.size(0) > 1 and p.size(1) > 1)
+        return preconditioned and not self.state[p].get("soap")
+
+    def _step_on_threads(self, device, streams, items) -> None:
+        """The initialising step: an eigensolve is tens of thousands of launches and the host does not run
+        that far ahead of the device, so parameters issued one after the other by one thread do not
+        overlap on the device however many streams they are spread over.  One host thread per side
+        stream takes every len(streams)-th parameter (the library calls release the interpreter lock)."""
+        failures = []
+
+        def worker(slot: int) -> None:
+            try:
+                with torch.cuda.device(device), torch.cuda.stream(streams[slot]), torch.no_grad():
+                    for p, group in items[slot::len(streams)]:
+                        self._step_parameter(p, group)
+            except BaseException as error:  # re-raised by the calling thread
+                failures.append(error)
+
+        threads = [threading.Thread(target=worker, args=(slot,), name=f"soap-init-{slot}") for slot in range(len(streams))]
+        for thread in threads:
+            thread.start()
+        for thread in threads:
+            thread.join()
+        if failures:
+            raise failures[0]
+
     @torch.no_grad()
     def step(self, closure=None):
         loss = None
@@ -172,10 +202,13 @@ class SOAP(torch.optim.Optimizer):
                 stream.wait_stream(main)
             # largest first, so the long steps start early and the small ones fill in
             order = sorted(range(len(items)), key=lambda i: -items[i][0].numel())
-            for slot, index in enumerate(order):
-                p, group = items[index]
-                with torch.cuda.stream(streams[slot % len(streams)]):
-                    self._step_parameter(p, group)
+            if any(self._uninitialised(items[index][0]) for index in order):
+                self._step_on_threads(device, streams, [items[index] for index in order])
+            else:
+                for slot, index in enumerate(order):
+                    p, group = items[index]
+                    with torch.cuda.stream(streams[slot % len(streams)]):
+                        self._step_parameter(p, group)
             for stream in streams:
                 main.wait_stream(stream)
         return loss

@@ -23,6 +23,7 @@ every intermediate stage exists to be dumped.
 from __future__ import annotations
 
 import math
+import threading
 from typing import Any, Literal, MutableMapping
 
 import torch
@@ -54,6 +55,18 @@ STATE_BUFFERS = (
     "momentum",
     "variance",
 )
+
+
+_SIDE_STREAMS: dict = {}
+
+
+def _side_stream(device, main) -> "torch.cuda.Stream":
+    """One extra stream (default priority) per device and calling stream, created on first use and
+    kept: callers that step parameters on several streams get a side stream for each of them."""
+    key = (torch.device(device), main.cuda_stream)
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=device)
+    return _SIDE_STREAMS[key]
 
 
 def _state_shapes(rows: int, columns: int) -> dict:
@@ -186,12 +199,49 @@ def soap_step(
 
     if initializing:
         update_preconditioners("")
-        for side, size in (("left", rows), ("right", columns)):
+
+        def initialize(side: str, size: int) -> None:
             with reporting_to(state["status"]):
                 initialize_basis_2d_block_cyclic_(
                     state[f"{side}_preconditioner"], state[f"{side}_basis"], state[f"{side}_work"],
                     torch.empty(size, dtype=torch.float32, device=device), size, block_size,
                     process_grid_shape, implementation=basis_implementation, elpa_binding=elpa_binding)
+
+        sides = (("left", rows), ("right", columns))
+        if elpa_binding is None and not profiling:
+            # The two eigensolves are independent: the smaller one runs on a side stream (default
+            # priority) forked from and joined back into the current one, so its latency-bound column
+            # steps fill the gaps of the larger one.  An eigensolve is tens of thousands of launches
+            # and the host does not run ahead of the device by that many, so the smaller one is
+            # enqueued by a helper thread while this one enqueues the larger one (the library calls
+            # release the interpreter lock).  Each solve's kernels and their order are what they are
+            # alone, so the bases are the same bit for bit.
+            small, large = sorted(sides, key=lambda item: item[1])
+            main = torch.cuda.current_stream(device)
+            side_stream = _side_stream(device, main)
+            side_stream.wait_stream(main)
+            failures = []
+
+            def enqueue_small() -> None:
+                try:
+                    with torch.cuda.device(device), torch.cuda.stream(side_stream), torch.no_grad():
+                        initialize(*small)
+                except BaseException as error:  # re-raised by the calling thread
+                    failures.append(error)
+
+            helper = threading.Thread(target=enqueue_small, name="soap-init-small-side")
+            helper.start()
+            try:
+                initialize(*large)
+            finally:
+                helper.join()
+                main.wait_stream(side_stream)
+            if failures:
+                raise failures[0]
+        else:
+            for side, size in sides:
+                initialize(side, size)
+        for side, _ in sides:
             _profile.dump(f"{side}_basis", profile_step, state[f"{side}_basis"])
         state["step"] = 0
         zero_update = torch.zeros_like(gradient)

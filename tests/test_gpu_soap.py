@@ -318,3 +318,24 @@ def test_nan_gradient_propagates_without_hanging(device):
                                        process_grid_shape=(1, 1), basis_refresh_interval=2)
         seen.append(bool(torch.isnan(update).any()))
     assert seen == [False, False, True, True, True, True]
+
+
+@pytest.mark.parametrize("shape,implementation", [((700, 1100), "elpa"), ((1100, 700), "eigh"), ((520, 520), "elpa")])
+def test_initial_eigensolves_side_by_side_equal_the_sequential_ones(shape, implementation, device):
+    """soap_step's first call runs its two eigensolves on two streams; each must give the basis that
+    the same solve gives alone on the current stream, bit for bit."""
+    from soap_tp_amd import ops
+    rows, columns = shape
+    gradient = torch.randn(rows, columns, generator=torch.Generator().manual_seed(SEED + 91)).to(device)
+    state = {}
+    soap_tp_amd.soap_step(gradient, state, global_shape=shape, shard_dim=1, block_size=128, process_grid_shape=(1, 1),
+                          basis_implementation=implementation)
+    torch.cuda.synchronize()
+    for side, size in (("left", rows), ("right", columns)):
+        basis = ops.allocate_2d_block_cyclic((size, size), 128, (1, 1), device=device)
+        work = ops.allocate_2d_block_cyclic((size, size), 128, (1, 1), device=device)
+        values = torch.empty(size, dtype=torch.float32, device=device)
+        ops.initialize_basis_2d_block_cyclic_(state[f"{side}_preconditioner"], basis, work, values, size, 128, (1, 1),
+                                              implementation=implementation)
+        assert torch.equal(basis, state[f"{side}_basis"]), side
+        assert torch.isfinite(basis).all()
