@@ -39,11 +39,21 @@ HBM_PEAK_GBS = 8000.0
 GRID = (1, 1)
 HYPER = dict(preconditioner_beta=0.95, beta1=0.95, beta2=0.95, eps=1e-8, basis_refresh_interval=10)
 
-# Memory bytes per launch of the rotation product (mean of the four launches of a step), from two
-# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of tests/native/abi_probe.bin, each scaled by what the
-# same counter reads for a layout copy of known size; summary under profiles/.  Keyed by shape; a shape
-# that has not been measured reports null.
-MEASURED_TRAFFIC_BYTES = {"4096x11008": 5.33e9}
+def measured_traffic_bytes(rows, columns):
+    """Memory bytes per launch of the rotation product (mean of the four launches of a step) for this
+    shape, read from the committed counter summary profiles/rotate_adam_rotate_<rows>x<columns>_memory_traffic.txt
+    (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE, of tests/native/abi_probe.bin, each scaled by what
+    the same counter reads for a layout copy of known size), with the file it came from; (None, None)
+    for a shape that has not been measured."""
+    import re
+    from pathlib import Path
+
+    path = Path(__file__).resolve().parent / "profiles" / f"rotate_adam_rotate_{rows}x{columns}_memory_traffic.txt"
+    if not path.exists():
+        return None, None
+    match = re.search(r"traffic per launch ([0-9.]+e[0-9]+) bytes", path.read_text())
+    return (float(match.group(1)), f"profiles/{path.name}") if match else (None, None)
+
 
 
 def gradient_pool(rows, columns, rank, count, device, seed0=42):
@@ -191,7 +201,7 @@ def checked_step(gradient, state, kwargs, hyper, step_function=None):
             "cpu_ms": cpu_ms}
 
 
-def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True, full_init=True):
+def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True, full_init=True, interval=10):
     """The CPU oracle on a bounded sample: `sample_plain_steps` steady-state steps and one refresh."""
     from oracle import soap_oracle as oracle
 
@@ -229,7 +239,6 @@ def cpu_baseline(shape, rank, sample_plain_steps=2, with_refresh=True, full_init
         start = time.perf_counter()
         oracle.eigh_descending(matrix, "elpa")
         init_ms[str(size)] = (time.perf_counter() - start) * 1e3
-    interval = HYPER["basis_refresh_interval"]
     per_step_ms = plain_ms + (refresh_ms / interval if refresh_ms is not None else 0.0)
     return {
         "value": 1e3 / per_step_ms, "unit": "steps/s", "cores": cores, "kind": "port",
@@ -395,6 +404,9 @@ def main():
     parser.add_argument("--shard-dim", type=int, default=1, choices=(0, 1),
                         help="shard_dim passed to the step (same mathematics on one rank; the reference's two Gram "
                              "code paths)")
+    parser.add_argument("--refresh-interval", type=int, default=HYPER["basis_refresh_interval"],
+                        help="steps between two basis refreshes of the main shape (the benchmark configurations use "
+                             "10, and 5 for 8192x3584)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-other-shapes", action="store_true")
     parser.add_argument("--cpu-small-init", action="store_true",
@@ -421,15 +433,17 @@ def main():
 
     if args.calibration_copies > 0:
         calibration_copies(rows, columns, args.calibration_copies, device)
+    if args.refresh_interval <= 0:
+        sys.exit("--refresh-interval must be positive.")
     main_run = run_schedule(args.shape, args.rank, args.steps, args.warmup, device, shard_dim=args.shard_dim,
-                            parity=True)
+                            interval=args.refresh_interval, parity=True)
     if not main_run["parity_check"]["ok"]:
         sys.exit(f"bench.py: the checked step disagrees with the CPU oracle: {main_run['parity_check']}")
     ms_per_step = main_run["total_ms"] / args.steps
     rotation_flops = 4.0 * rows * columns * (rows + columns)
     gram_flops = 1.0 * rows * columns * (rows + columns)
     achieved = rotation_flops / (main_run["rotate_ms"] * 1e-3) / 1e12
-    traffic = MEASURED_TRAFFIC_BYTES.get(f"{rows}x{columns}")
+    traffic, traffic_source = measured_traffic_bytes(rows, columns)
     line = {
         "metric": "SOAP steps/sec per param shape (1 GPU)",
         "value": args.steps / (main_run["total_ms"] * 1e-3),
@@ -447,7 +461,7 @@ def main():
             "workload": f"{rows}x{columns} fp32 parameter, rank-{args.rank} low-rank-plus-noise gradients "
                         f"(log-uniform spectrum 1e-4..1e-1, noise std 1e-4), world_size 1, shard_dim {args.shard_dim}, "
                         f"block_size 128, "
-                        f"refresh every {HYPER['basis_refresh_interval']} steps, beta1=beta2=shampoo_beta=0.95, "
+                        f"refresh every {args.refresh_interval} steps, beta1=beta2=shampoo_beta=0.95, "
                         "eps=1e-8, basis_implementation=elpa (fp64 eigensolve)",
             "schedule": f"{args.warmup} warm-up calls (initialisation + {args.warmup - 1} steps), then {args.steps} "
                         f"timed calls of soap_step ({main_run['refreshes']} of them refresh the bases)",
@@ -473,7 +487,8 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
             "traffic": traffic,
-            "traffic_unit": "bytes per launch (L2 fills + writes; compulsory 0.82e9)",
+            "traffic_unit": "bytes per launch (L2 fills + writes; compulsory 0.82e9 at 4096x11008)",
+            "traffic_source": traffic_source,
             "flops_per_step": rotation_flops,
             "avg_launch_ms": main_run["rotate_ms"] / 4.0,
             "gram_pair_tflops_syrk_convention": gram_flops / (main_run["gram_ms"] * 1e-3) / 1e12,
@@ -501,7 +516,7 @@ def main():
     if not args.no_layer:
         line["layer"] = run_layer(device)
     if not args.no_cpu_baseline:
-        baseline = cpu_baseline(args.shape, args.rank, full_init=not args.cpu_small_init)
+        baseline = cpu_baseline(args.shape, args.rank, full_init=not args.cpu_small_init, interval=args.refresh_interval)
         gpu_ms = gpu_eigensolve_ms([int(size) for size in baseline["init_eigensolve_ms_by_size"]], args.rank, device)
         baseline["gpu_eigensolve_ms_by_size"] = gpu_ms
         baseline["eigensolve_speedup_by_size"] = {

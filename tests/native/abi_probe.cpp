@@ -4,7 +4,8 @@
 //   abi_probe qr n          QR of a pseudo-random n x n matrix (library-owned workspace), Q checked on the host
 //   abi_probe eigh n        fp64 eigendecomposition of a symmetric n x n matrix, checked on the host
 //   abi_probe eigh n [timed] two-stage   the eigh modes with the two-stage tridiagonalisation
-//   abi_probe qr n [timed] two-level    the qr modes with 256-wide block reflectors only (no super-blocks)
+//   abi_probe qr n [timed] two-level|three-level   the qr modes with the blocking fixed: 256-wide block reflectors
+//                               only, or 1024-column super-blocks (left to the library: three levels up to n = 4096)
 //   abi_probe qr|eigh n timed   the same call four times, the last three timed, no host check (the
 //                               check is cubic on one core: minutes at n = 11008)
 //
@@ -170,8 +171,9 @@ int main(int argc, char** argv) {
     ABI_OK(soapmi_set_option("eigh_algorithm", 2));
     --argc;
   }
-  if (argc >= 4 && std::string(argv[1]) == "qr" && std::string(argv[argc - 1]) == "two-level") {
-    ABI_OK(soapmi_set_option("qr_super_block", 256));
+  if (argc >= 4 && std::string(argv[1]) == "qr" &&
+      (std::string(argv[argc - 1]) == "two-level" || std::string(argv[argc - 1]) == "three-level")) {
+    ABI_OK(soapmi_set_option("qr_super_block", std::string(argv[argc - 1]) == "two-level" ? 256 : 1024));
     --argc;
   }
   const bool timed_only = argc == 4 && std::string(argv[3]) == "timed";
