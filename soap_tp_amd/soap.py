@@ -181,7 +181,7 @@ def soap_step(
     _profile.dump("gradient", profile_step, gradient)
 
     def update_preconditioners(suffix: str) -> None:
-        if slate_binding is None and not profiling and not initializing:
+        if slate_binding is None and not profiling:
             _fused_gram_pair(gradient, state, rows, columns, preconditioner_beta, mirror)
             return
         update_left_preconditioner_2d_block_cyclic_(
