@@ -290,6 +290,18 @@ def test_config_4096x4096_full_schedule(device, monkeypatch):
         assert identity_error.abs().max().item() <= 1e-4
 
 
+def test_config_4096x11008_two_refresh_cycles(device, monkeypatch):
+    """The third benchmark configuration at its real cadence: 4096 x 11008, rank 128, a refresh every 10,
+    twenty steps after the initialising call (two refreshes; the configuration's full fifty would keep the
+    CPU oracle busy for several minutes).  Every iteration's update against the oracle given the
+    device's bases; moments and Gram matrices at the end."""
+    shape = (4096, 11008)
+    gradients = [oracle.low_rank_plus_noise(*shape, 128, seed=SEED + 700 + t) for t in range(21)]
+    updates, state, bases = run_recorded(gradients, device, monkeypatch, interval=10)
+    assert sorted(bases) == [0, 10, 20]
+    assert_conditional_parity(gradients, updates, state, bases, 10)
+
+
 LAYER = (("q", (4096, 4096)), ("k", (4096, 4096)), ("v", (4096, 4096)), ("o", (4096, 4096)),
          ("gate", (4096, 14336)), ("up", (4096, 14336)), ("down", (14336, 4096)))
 
