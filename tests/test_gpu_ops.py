@@ -546,6 +546,49 @@ def test_a_failed_factorisation_is_attributed_to_its_state(device):
     assert not _native.device_error_flag(clear=True)  # the device-wide word was never involved
 
 
+def test_status_word_through_the_c_abi(device):
+    """soapmi_set_status_word called directly: while a caller-owned word (pinned host memory) is set for this
+    thread, a factorisation that gives up raises that word and leaves the device-wide one alone; after
+    NULL the device-wide word is back in charge.  (Spin limit 0 makes the kernels give up without
+    waiting; every kernel exits normally.)"""
+    from soap_tp_amd import _native
+    size = 700
+    matrix = make_matrix(size, size, seed=SEED + 83)
+    word = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+    stream = torch.cuda.current_stream().cuda_stream
+    need = _native.library().soapmi_qr_workspace_bytes(size)
+    work = torch.empty(need, dtype=torch.uint8, device=device)
+
+    def qr():
+        a, q = column_major(matrix, device), torch.empty(size, size, device=device).T
+        _native.call("soapmi_qr_f32", a.data_ptr(), q.data_ptr(), size, a.stride(1), q.stride(1), work.data_ptr(), need,
+                     stream)
+        torch.cuda.synchronize()
+        return q
+
+    assert not _native.device_error_flag(clear=True)
+    try:
+        _native.call("soapmi_set_option", b"message_spin_limit", 0)
+        _native.call("soapmi_set_status_word", word.data_ptr())
+        with_word = qr()
+        _native.call("soapmi_set_status_word", 0)
+        assert not _native.device_error_flag(clear=True)  # whatever happened went to the caller's word
+        assert bool(word[0] != 0) == bool(torch.isnan(with_word).any())
+        without_word = qr()
+        assert _native.device_error_flag(clear=True) == bool(torch.isnan(without_word).any())
+    finally:
+        _native.call("soapmi_set_status_word", 0)
+        _native.call("soapmi_set_option", b"message_spin_limit", 1 << 22)
+        _native.device_error_flag(clear=True)
+    word.zero_()
+    _native.call("soapmi_set_status_word", word.data_ptr())
+    try:
+        clean = qr()
+    finally:
+        _native.call("soapmi_set_status_word", 0)
+    assert int(word[0]) == 0 and relative_l2(clean.cpu(), oracle.householder_qr(matrix)) <= 5e-5
+
+
 @pytest.mark.parametrize("budget", [256, 20])
 def test_factorisations_on_several_streams_share_the_chip_safely(budget, device):
     """Four QR factorisations of 4096 x 4096 matrices (16 workgroups each in their panel kernels) and
