@@ -6,6 +6,11 @@
 //   abi_probe eigh n [timed] two-stage   the eigh modes with the two-stage tridiagonalisation
 //   abi_probe qr n [timed] two-level|three-level   the qr modes with the blocking fixed: 256-wide block reflectors
 //                               only, or 1024-column super-blocks (left to the library: three levels up to n = 4096)
+//   abi_probe burst             how the rate of one MFMA product (soapmi_gemm_f32, 11008 x 9984 x 1024, C -= A B) depends on what
+//                               the device did just before: a steady stream of such products, the first ones after
+//                               300 ms idle, and two of them alternating with 2.5 ms of idle, of tiny launches and
+//                               of device-to-device copies (the pattern of a factorisation whose products sit
+//                               between latency-bound panel phases)
 //   abi_probe qr|eigh n timed   the same call four times, the last three timed, no host check (the
 //                               check is cubic on one core: minutes at n = 11008)
 //
@@ -22,6 +27,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <unistd.h>
 #include <string>
 #include <vector>
 
@@ -165,7 +171,83 @@ static int check_eigh(int64_t n, bool timed_only) {
   return 0;
 }
 
+// (The probe is built for the host only: it launches no kernels of its own.  Device buffers are filled from the
+// host; the "tiny launch" is the library's layout copy of an 8 x 8 matrix.)
+static int check_burst() {
+  const int64_t M = 11008, N = 9984, K = 1024;
+  float *a, *b, *c, *tiny;
+  HIP_OK(hipMalloc((void**)&a, M * K * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&b, K * N * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&c, 2 * M * N * sizeof(float)));  // second half: target of the filler copies
+  HIP_OK(hipMalloc((void**)&tiny, 512));
+  HIP_OK(hipMemset(tiny, 0, 512));
+  {
+    std::vector<float> host((size_t)M * N);
+    for (size_t i = 0; i < host.size(); ++i) host[i] = host_value(i);
+    HIP_OK(hipMemcpy(c, host.data(), (size_t)M * N * sizeof(float), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(a, host.data(), (size_t)M * K * sizeof(float), hipMemcpyHostToDevice));
+    for (size_t i = 0; i < (size_t)K * N; ++i) host[i] *= 1e-3f;
+    HIP_OK(hipMemcpy(b, host.data(), (size_t)K * N * sizeof(float), hipMemcpyHostToDevice));
+  }
+  const double flops = 2.0 * (double)M * (double)N * (double)K;
+  auto product = [&]() { return soapmi_gemm_f32(0, 0, M, N, K, -1.0f, a, M, b, K, 1.0f, c, M, nullptr); };
+  hipEvent_t ev[64];
+  for (auto& e : ev) HIP_OK(hipEventCreate(&e));
+  auto report = [&](const char* what, double us) {
+    std::printf("%-58s %7.0f us  %6.1f TFLOP/s\n", what, us, flops / us / 1e6);
+  };
+  // 1. after idle, then a steady stream
+  for (int i = 0; i < 40; ++i) ABI_OK(product());
+  HIP_OK(hipDeviceSynchronize());
+  usleep(300000);
+  for (int i = 0; i < 63; ++i) {
+    HIP_OK(hipEventRecord(ev[i], nullptr));
+    ABI_OK(product());
+  }
+  HIP_OK(hipEventRecord(ev[63], nullptr));
+  HIP_OK(hipDeviceSynchronize());
+  double first = 0.0, steady = 0.0;
+  for (int i = 0; i < 63; ++i) {
+    float ms = 0.0f;
+    HIP_OK(hipEventElapsedTime(&ms, ev[i], ev[i + 1]));
+    if (i < 3) first += ms * 1000.0 / 3.0;
+    if (i >= 43) steady += ms * 1000.0 / 20.0;
+  }
+  report("first three products after 300 ms idle (mean)", first);
+  report("products 44..63 of the same stream (mean)", steady);
+  // 2. two products alternating with 2.5 ms of something else; the last of 14 rounds is reported
+  const char* names[3] = {"two products after 2.5 ms idle, 14th round", "two products after 500 tiny launches, 14th round",
+                          "two products after 12 device-to-device copies, 14th round"};
+  for (int mode = 0; mode < 3; ++mode) {
+    float ms = 0.0f;
+    for (int round = 0; round < 14; ++round) {
+      if (mode == 0) {
+        HIP_OK(hipDeviceSynchronize());
+        usleep(2500);
+      } else if (mode == 1) {
+        for (int i = 0; i < 500; ++i) ABI_OK(soapmi_row_major_to_col_major_f32(tiny, 8, tiny + 32, 8, 8, 8, nullptr));
+      } else {
+        for (int i = 0; i < 12; ++i)
+          HIP_OK(hipMemcpyAsync(c + M * N, c + M * N / 2, (size_t)M * N * 2, hipMemcpyDeviceToDevice, nullptr));
+      }
+      HIP_OK(hipEventRecord(ev[0], nullptr));
+      ABI_OK(product());
+      ABI_OK(product());
+      HIP_OK(hipEventRecord(ev[1], nullptr));
+      HIP_OK(hipDeviceSynchronize());
+      HIP_OK(hipEventElapsedTime(&ms, ev[0], ev[1]));
+    }
+    report(names[mode], ms * 500.0);
+    for (int i = 0; i < 30; ++i) ABI_OK(product());  // back to the steady state before the next pattern
+    HIP_OK(hipDeviceSynchronize());
+  }
+  hipFree(a); hipFree(b); hipFree(c); hipFree(tiny);
+  std::printf("ok\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
+  if (argc == 2 && std::string(argv[1]) == "burst") return check_burst();
   // a trailing "two-stage" selects the two-stage tridiagonalisation for the eigh modes
   if (argc >= 4 && std::string(argv[1]) == "eigh" && std::string(argv[argc - 1]) == "two-stage") {
     ABI_OK(soapmi_set_option("eigh_algorithm", 2));
