@@ -30,6 +30,7 @@ namespace soapmi {
 constexpr int kTrdNb = 32;        // panel width
 constexpr int kTrdTile = 128;     // tile edge of the matrix-vector product
 constexpr int kTrdMaxWg = 128;    // workgroups of the fused column kernel (256 rows each)
+constexpr double kTrdReverseAboveBytes = 320.0 * 1024 * 1024;  // see trd_symv_kernel's `reverse`
 constexpr int kTrdWideBelow = 256;  // tiles up to which the matrix-vector kernel runs 512 threads per tile (one tile per compute unit)
 
 template <typename T>
@@ -392,7 +393,8 @@ __global__ __launch_bounds__(256) void trd_column_kernel(T* __restrict__ A, int6
 // a compute unit holds one such workgroup), and QS = 1, three tiles per compute unit, above.
 template <typename T, int QS>
 __global__ __launch_bounds__(256 * QS) void trd_symv_kernel(const T* __restrict__ A, int64_t lda, int n, int j,
-                                                            const T* __restrict__ v, T* __restrict__ y_part) {
+                                                            const T* __restrict__ v, T* __restrict__ y_part,
+                                                            int reverse) {
   constexpr int TS = kTrdTile;
   __shared__ T s_v[TS];
   __shared__ T s_direct[2 * QS][TS];
@@ -403,7 +405,12 @@ __global__ __launch_bounds__(256 * QS) void trd_symv_kernel(const T* __restrict_
   // address arithmetic to the scalar unit
   const int row = tid & (TS - 1), half = __builtin_amdgcn_readfirstlane(tid >> 7);
   const int o = j + 1;
-  const int t = blockIdx.x;
+  // Workgroups start in the order of their ids.  Every other column walks the tiles backwards: the
+  // tiles a launch touches last are the ones most likely still held by the 256 MB memory-side cache
+  // when the next column's launch, whose tiles are the same memory shifted by one row and column,
+  // begins with them.  (Walking forwards every time, a matrix larger than that cache evicts the
+  // head of the walk before the next launch comes back to it.)
+  const int t = reverse ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
   int rb = (int)((sqrtf(8.0f * (float)t + 1.0f) - 1.0f) * 0.5f);
   while (rb * (rb + 1) / 2 > t) --rb;
   while ((rb + 1) * (rb + 2) / 2 <= t) ++rb;
@@ -497,12 +504,16 @@ static inline int sytrd_lower(hipStream_t s, T* A, int64_t lda, int n, T* d, T* 
       const int i = j - p;
       const int nt = n - j - 1;
       const int nb = (int)ceil_div64(nt, kTrdTile);
+      // (backwards on every other column while the triangle that is read is larger than the memory-side
+      // cache: measured 662 -> 646 ms at n = 11008 and 1297 -> 1263 ms at 14336 in fp64; below that size
+      // it costs 1 to 2 %)
+      const int reverse = ((j & 1) != 0 && (double)nt * (double)nt * 0.5 * sizeof(T) > kTrdReverseAboveBytes) ? 1 : 0;
       if (nb * (nb + 1) / 2 <= kTrdWideBelow)
         hipLaunchKernelGGL((trd_symv_kernel<T, 2>), dim3(nb * (nb + 1) / 2), dim3(512), 0, s, A, lda, n, j,
-                           ws.vc + (int64_t)i * ldw, ws.y_part);
+                           ws.vc + (int64_t)i * ldw, ws.y_part, reverse);
       else
         hipLaunchKernelGGL((trd_symv_kernel<T, 1>), dim3(nb * (nb + 1) / 2), dim3(256), 0, s, A, lda, n, j,
-                           ws.vc + (int64_t)i * ldw, ws.y_part);
+                           ws.vc + (int64_t)i * ldw, ws.y_part, reverse);
       grid = (int)ceil_div64(nt, 256);
       const int do_next = (j + 1 < pe) ? 1 : 0;
       hipLaunchKernelGGL((trd_column_kernel<T>), dim3(grid), dim3(256), 0, s, A, lda, n, p, j, 1, do_next, ws.vc, ws.vc2,
