@@ -11,7 +11,8 @@
  *     synchronising;
  *   - `workspace` may be NULL: the library then uses a per-device buffer it grows on demand
  *     (not safe for concurrent use from several streams); otherwise it must hold at least
- *     the bytes reported by the matching *_workspace_bytes query;
+ *     the bytes reported by the matching *_workspace_bytes query (the sizes do not depend on
+ *     soapmi_set_option: they cover both tridiagonalisations and both QR blockings);
  *   - return value 0 = success; <0 = error (SOAPMI_INVALID_ARGUMENT is the analogue of the
  *     std::invalid_argument the reference bindings throw, SOAPMI_RUNTIME_ERROR of
  *     std::runtime_error); soapmi_last_error() returns the message of the calling thread's
