@@ -168,7 +168,10 @@ def soap_step(
     raise_on_state_error(state)
     raise_on_device_error(device)
     initializing = "left_basis" not in state
-    if "status" not in state:  # (a state restored from a checkpoint comes without one)
+    status = state.get("status")
+    if not (isinstance(status, Tensor) and status.dtype == torch.int32 and status.numel() >= 1 and status.is_pinned()):
+        # (a state restored from a checkpoint comes without one; a deep copy of a state has one that
+        # is no longer pinned memory, which a kernel could not write to)
         state["status"] = new_status_word()
 
     if initializing:

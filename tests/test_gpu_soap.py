@@ -339,3 +339,22 @@ def test_initial_eigensolves_side_by_side_equal_the_sequential_ones(shape, imple
                                               implementation=implementation)
         assert torch.equal(basis, state[f"{side}_basis"]), side
         assert torch.isfinite(basis).all()
+
+
+def test_a_deep_copied_state_keeps_working(device):
+    """copy.deepcopy turns the state's pinned failure word into ordinary host memory; soap_step must
+    replace it instead of handing a kernel an address it cannot write to."""
+    import copy
+    shape = (300, 520)
+    generator = torch.Generator().manual_seed(SEED + 93)
+    gradients = [torch.randn(*shape, generator=generator).to(device) for _ in range(5)]
+    kwargs = dict(global_shape=shape, shard_dim=1, block_size=128, process_grid_shape=(1, 1), basis_refresh_interval=2)
+    state = {}
+    for gradient in gradients[:2]:
+        soap_tp_amd.soap_step(gradient, state, **kwargs)
+    clone = copy.deepcopy(state)
+    for gradient in gradients[2:]:  # steps 2 and 4 refresh
+        a = soap_tp_amd.soap_step(gradient, state, **kwargs)
+        b = soap_tp_amd.soap_step(gradient, clone, **kwargs)
+        assert torch.equal(a, b)
+    assert clone["status"].is_pinned() and int(clone["status"][0]) == 0
